@@ -1,0 +1,323 @@
+// Row-wise and element-wise kernels: embedding gather, RMS norms joined to the
+// residual stream, gated activation, soft cap, rotary encoding with the write
+// into the paged cache, dtype conversion and seeded random fill.
+//
+// Formulas follow the reference's kernels, which are fp16 strings compiled at
+// run time (zse-engine/zse_engine/orchestrator/kernels.py): gather to an fp32
+// stream :1789-1806, rsqrt(sum/H + eps) :1435-1465, rotate-half pairs
+// :264-297, gelu-tanh gate :1678-1697, cap*tanh(x/cap) :1714-1727, the scatter
+// of K and V into pages :961-1012.
+#include "common.h"
+
+thread_local std::string zk_error;
+int zk_fail(const char* msg) {
+  zk_error = msg;
+  return -1;
+}
+int zk_launch_status(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    zk_error = std::string(what) + ": " + hipGetErrorString(e);
+    return (int)e;
+  }
+  return 0;
+}
+
+// ------------------------------------------------------------------ embedding
+
+template <typename W>
+__global__ void embed_kernel(const W* __restrict__ table, const int* __restrict__ tokens,
+                             float* __restrict__ out, float scale, int H, int V) {
+  const int t = blockIdx.x;
+  int tok = tokens[t];
+  tok = tok < 0 ? 0 : (tok >= V ? V - 1 : tok);
+  const W* row = table + (size_t)tok * H;
+  float* o = out + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32(row[i]) * scale;
+}
+
+// ------------------------------------------------------------------ norms
+
+__device__ __forceinline__ float gain(const float* w, int i, int unit_offset) {
+  return unit_offset ? 1.f + w[i] : w[i];
+}
+
+// out[r] = N(x[rows ? rows[r] : r])
+template <typename TIn>
+__global__ void rmsnorm_kernel(const TIn* __restrict__ x, const int* __restrict__ rows,
+                               const float* __restrict__ w, act_t* __restrict__ out, float eps,
+                               int unit_offset, int H) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  const TIn* xr = x + (size_t)src * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = to_f32(xr[i]);
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float rs = rsqrtf(ss / (float)H + eps);
+  act_t* o = out + (size_t)r * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x)
+    o[i] = from_f32<act_t>(to_f32(xr[i]) * rs * gain(w, i, unit_offset));
+}
+
+// h += N_post(sub)  (w_post null: h += sub);  then, if w_next: out = N_next(h)
+__global__ void norm_add_norm_kernel(const act_t* __restrict__ sub, const float* __restrict__ w_post,
+                                     float eps_post, int uo_post, float* __restrict__ h,
+                                     const float* __restrict__ w_next, float eps_next, int uo_next,
+                                     act_t* __restrict__ out, int H) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const act_t* s = sub + (size_t)r * H;
+  float* hr = h + (size_t)r * H;
+  float rs = 1.f;
+  if (w_post) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+      float v = to_f32(s[i]);
+      ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    rs = rsqrtf(ss / (float)H + eps_post);
+  }
+  float ss2 = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = to_f32(s[i]);
+    if (w_post) v = v * rs * gain(w_post, i, uo_post);
+    v = hr[i] + v;
+    hr[i] = v;
+    ss2 += v * v;
+  }
+  if (!w_next) return;
+  ss2 = block_sum(ss2, red);
+  const float rs2 = rsqrtf(ss2 / (float)H + eps_next);
+  act_t* o = out + (size_t)r * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x)  // each thread re-reads what it wrote
+    o[i] = from_f32<act_t>(hr[i] * rs2 * gain(w_next, i, uo_next));
+}
+
+// ------------------------------------------------------------------ gated activation
+
+__device__ __forceinline__ float gelu_tanh(float g) {
+  const float k = 0.7978845608028654f;
+  return 0.5f * g * (1.0f + tanhf(k * (g + 0.044715f * g * g * g)));
+}
+__device__ __forceinline__ float silu(float g) { return g / (1.0f + expf(-g)); }
+
+// gu: [T, 2I], gate in columns [0, I), up in [I, 2I)
+__global__ void gated_act_kernel(const act_t* __restrict__ gu, act_t* __restrict__ out, int I,
+                                 int act) {
+  const int t = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= I) return;
+  const float g = to_f32(gu[(size_t)t * 2 * I + i]);
+  const float u = to_f32(gu[(size_t)t * 2 * I + I + i]);
+  const float a = act == 0 ? gelu_tanh(g) : silu(g);
+  out[(size_t)t * I + i] = from_f32<act_t>(a * u);
+}
+
+__global__ void softcap_kernel(float* __restrict__ z, size_t n, float cap) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) z[i] = cap * tanhf(z[i] / cap);
+}
+
+// ------------------------------------------------------------------ rotary + cache write
+
+// qkv: [T, (nh + 2 nkv) hd] rows of [q | k | v].  q is rotated in place; k is
+// rotated and stored, v is stored, at slot = page * bs + offset of the token
+// (slot < 0: nothing stored).  Cache layout per layer: [page][kv head][bs][hd].
+__global__ void rope_cache_write_kernel(act_t* __restrict__ qkv, const int* __restrict__ positions,
+                                        const int* __restrict__ slot_map,
+                                        const float* __restrict__ inv_freq, int rotary_dim,
+                                        act_t* __restrict__ kcache, act_t* __restrict__ vcache,
+                                        int nh, int nkv, int hd, int bs) {
+  const int t = blockIdx.x;
+  const int head = blockIdx.y;  // [0,nh): q; [nh, nh+nkv): k; [nh+nkv, nh+2nkv): v
+  act_t* src = qkv + (size_t)t * (nh + 2 * nkv) * hd + (size_t)head * hd;
+  const float pos = (float)positions[t];
+  const int half = rotary_dim / 2;
+  const int slot = slot_map ? slot_map[t] : -1;
+  act_t* dst = nullptr;
+  if (head >= nh && slot >= 0) {
+    const int kvh = (head - nh) % nkv;
+    act_t* base = head < nh + nkv ? kcache : vcache;
+    const size_t page = slot / bs, off = slot % bs;
+    dst = base + ((page * nkv + kvh) * bs + off) * hd;
+  }
+  if (head < nh + nkv) {
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+      const float ang = pos * inv_freq[i];
+      float sn, cs;
+      sincosf(ang, &sn, &cs);
+      const float a = to_f32(src[i]), b = to_f32(src[i + half]);
+      const act_t ra = from_f32<act_t>(a * cs - b * sn), rb = from_f32<act_t>(b * cs + a * sn);
+      if (head < nh) {
+        src[i] = ra;
+        src[i + half] = rb;
+      } else if (dst) {
+        dst[i] = ra;
+        dst[i + half] = rb;
+      }
+    }
+    if (head >= nh && dst)
+      for (int i = rotary_dim + threadIdx.x; i < hd; i += blockDim.x) dst[i] = src[i];
+  } else if (dst) {
+    for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[i] = src[i];
+  }
+}
+
+// ------------------------------------------------------------------ conversion, fill
+
+// src_tag: 0 = float32, 1 = bfloat16, 2 = float16
+template <typename D>
+__global__ void convert_kernel(const void* __restrict__ src, int src_tag, D* __restrict__ dst,
+                               size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float v;
+  if (src_tag == 0) v = ((const float*)src)[i];
+  else if (src_tag == 1) v = (float)((const __bf16*)src)[i];
+  else v = (float)((const _Float16*)src)[i];
+  dst[i] = from_f32<D>(v);
+}
+
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+// Normal(mean, std) values as a pure function of (seed, stream, element index).
+template <typename D>
+__global__ void fill_normal_kernel(D* __restrict__ dst, size_t n, uint64_t seed, uint64_t stream,
+                                   float mean, float std) {
+  size_t pair = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t i = pair * 2;
+  if (i >= n) return;
+  uint64_t r = mix64(mix64(seed ^ (stream * 0xD1342543DE82EF95ull)) + pair);
+  const float u1 = ((float)(uint32_t)(r >> 40) + 1.0f) * (1.0f / 16777216.0f);  // (0, 1]
+  const float u2 = (float)(uint32_t)((r >> 8) & 0xFFFFFF) * (1.0f / 16777216.0f);
+  const float rad = sqrtf(-2.0f * logf(u1));
+  float sn, cs;
+  sincosf(6.283185307179586f * u2, &sn, &cs);
+  dst[i] = from_f32<D>(mean + std * rad * cs);
+  if (i + 1 < n) dst[i + 1] = from_f32<D>(mean + std * rad * sn);
+}
+
+__global__ void zero_kernel(uint32_t* __restrict__ p, size_t n_words) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_words) p[i] = 0u;
+}
+
+// ------------------------------------------------------------------ C interface
+
+extern "C" {
+
+const char* zk_last_error() { return zk_error.c_str(); }
+int zk_act_is_bf16() { return ZSE_ACT_BF16; }
+
+int zk_embed(const void* table, const int* tokens, float* out, float scale, int T, int H, int V,
+             void* stream) {
+  ZK_REQUIRE(T >= 0 && H > 0 && V > 0, "zk_embed: bad sizes");
+  if (T == 0) return 0;
+  embed_kernel<act_t><<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)table, tokens, out, scale, H, V);
+  return zk_launch_status("zk_embed");
+}
+
+// x_is_f32: input rows are the float residual stream, else activations.
+int zk_rmsnorm(const void* x, int x_is_f32, const int* rows, const float* w, void* out, float eps,
+               int unit_offset, int R, int H, void* stream) {
+  ZK_REQUIRE(R >= 0 && H > 0, "zk_rmsnorm: bad sizes");
+  if (R == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (x_is_f32)
+    rmsnorm_kernel<float><<<R, 256, 0, s>>>((const float*)x, rows, w, (act_t*)out, eps, unit_offset, H);
+  else
+    rmsnorm_kernel<act_t><<<R, 256, 0, s>>>((const act_t*)x, rows, w, (act_t*)out, eps, unit_offset, H);
+  return zk_launch_status("zk_rmsnorm");
+}
+
+int zk_norm_add_norm(const void* sub, const float* w_post, float eps_post, int uo_post, float* h,
+                     const float* w_next, float eps_next, int uo_next, void* out, int T, int H,
+                     void* stream) {
+  ZK_REQUIRE(T >= 0 && H > 0, "zk_norm_add_norm: bad sizes");
+  ZK_REQUIRE(w_next == nullptr || out != nullptr, "zk_norm_add_norm: next norm without output");
+  if (T == 0) return 0;
+  norm_add_norm_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)sub, w_post, eps_post, uo_post, h,
+                                                           w_next, eps_next, uo_next, (act_t*)out, H);
+  return zk_launch_status("zk_norm_add_norm");
+}
+
+// act: 0 = gelu_tanh, 1 = silu
+int zk_gated_act(const void* gu, void* out, int T, int I, int act, void* stream) {
+  ZK_REQUIRE(T >= 0 && I > 0 && (act == 0 || act == 1), "zk_gated_act: bad arguments");
+  ZK_REQUIRE(T <= 65535, "zk_gated_act: more than 65535 rows");
+  if (T == 0) return 0;
+  dim3 grid((I + 255) / 256, T);
+  gated_act_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)gu, (act_t*)out, I, act);
+  return zk_launch_status("zk_gated_act");
+}
+
+int zk_softcap(float* z, size_t n, float cap, void* stream) {
+  ZK_REQUIRE(cap > 0.f, "zk_softcap: cap must be positive");
+  if (n == 0) return 0;
+  ZK_REQUIRE((n + 255) / 256 < 2147483647ull, "zk_softcap: too many elements");
+  softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(z, n, cap);
+  return zk_launch_status("zk_softcap");
+}
+
+int zk_rope_cache_write(void* qkv, const int* positions, const int* slot_map, const float* inv_freq,
+                        int rotary_dim, void* kcache, void* vcache, int T, int nh, int nkv, int hd,
+                        int bs, void* stream) {
+  ZK_REQUIRE(T >= 0 && nh > 0 && nkv >= 0 && hd > 0 && bs > 0, "zk_rope_cache_write: bad sizes");
+  ZK_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && rotary_dim % 2 == 0,
+             "zk_rope_cache_write: rotary_dim must be even and at most head_dim");
+  ZK_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "zk_rope_cache_write: no frequency table");
+  ZK_REQUIRE(nh + 2 * nkv <= 65535, "zk_rope_cache_write: too many heads");
+  if (T == 0) return 0;
+  dim3 grid(T, nh + 2 * nkv);
+  rope_cache_write_kernel<<<grid, 64, 0, (hipStream_t)stream>>>((act_t*)qkv, positions, slot_map, inv_freq,
+                                                                rotary_dim, (act_t*)kcache,
+                                                                (act_t*)vcache, nh, nkv, hd, bs);
+  return zk_launch_status("zk_rope_cache_write");
+}
+
+// dst_kind: 0 = float32, 1 = the library's activation type
+int zk_convert(const void* src, int src_tag, void* dst, int dst_kind, size_t n, void* stream) {
+  ZK_REQUIRE(src_tag >= 0 && src_tag <= 2 && (dst_kind == 0 || dst_kind == 1), "zk_convert: bad tags");
+  if (n == 0) return 0;
+  ZK_REQUIRE((n + 255) / 256 < 2147483647ull, "zk_convert: too many elements");
+  unsigned g = (unsigned)((n + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (dst_kind == 0) convert_kernel<float><<<g, 256, 0, s>>>(src, src_tag, (float*)dst, n);
+  else convert_kernel<act_t><<<g, 256, 0, s>>>(src, src_tag, (act_t*)dst, n);
+  return zk_launch_status("zk_convert");
+}
+
+int zk_fill_normal(void* dst, int dst_kind, size_t n, uint64_t seed, uint64_t stream_id, float mean,
+                   float std, void* stream) {
+  ZK_REQUIRE(dst_kind == 0 || dst_kind == 1, "zk_fill_normal: bad dst kind");
+  if (n == 0) return 0;
+  size_t pairs = (n + 1) / 2;
+  ZK_REQUIRE((pairs + 255) / 256 < 2147483647ull, "zk_fill_normal: too many elements");
+  unsigned g = (unsigned)((pairs + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (dst_kind == 0) fill_normal_kernel<float><<<g, 256, 0, s>>>((float*)dst, n, seed, stream_id, mean, std);
+  else fill_normal_kernel<act_t><<<g, 256, 0, s>>>((act_t*)dst, n, seed, stream_id, mean, std);
+  return zk_launch_status("zk_fill_normal");
+}
+
+// Clears ``nbytes`` (a multiple of 4) with a kernel, so that it may be captured in a graph.
+int zk_zero(void* p, size_t nbytes, void* stream) {
+  ZK_REQUIRE(nbytes % 4 == 0, "zk_zero: size must be a multiple of 4 bytes");
+  if (nbytes == 0) return 0;
+  size_t n = nbytes / 4;
+  ZK_REQUIRE((n + 255) / 256 < 2147483647ull, "zk_zero: too many bytes");
+  zero_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>((uint32_t*)p, n);
+  return zk_launch_status("zk_zero");
+}
+
+}  // extern "C"

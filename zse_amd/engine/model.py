@@ -1,0 +1,77 @@
+"""A model: the parts a plan names, built, loaded and run in the plan's order."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+from .. import parts as _parts  # noqa: F401  (registers the built-in part kinds)
+from ..config.plan import ModelPlan
+from ..parts.base import PagedKV, Part, StateNeed, TensorReq, build_part, walk
+from ..runtime.device import F32, Tensor
+
+
+@dataclass
+class CallCache:
+    """What one entry of the execution order keeps between steps."""
+    need: object = None              # PagedKV | StateNeed | None
+    group: Optional[int] = None      # cache group of a paged need
+    k: Optional[Tensor] = None       # [pages, kv heads, page size, head dim]
+    v: Optional[Tensor] = None
+    state_offset: int = 0            # byte offset inside a request's state slot
+    state_bytes: int = 0
+
+
+class Model:
+    def __init__(self, plan: ModelPlan):
+        self.plan = plan
+        self.embedding = build_part("embedding", plan.embedding)
+        self.blocks = [build_part("block", b) for b in plan.layers]
+        self.final_norm = build_part("norm", plan.final_norm)
+        self.head = build_part("head", plan.head)
+        for i, call in enumerate(plan.order):
+            if not (0 <= call.layer < len(self.blocks)):
+                raise ValueError(f"order entry {i} names layer {call.layer}, which does not exist")
+            if call.cache_of is not None and not (0 <= call.cache_of < i):
+                raise ValueError(f"order entry {i} reads the cache of entry {call.cache_of}, "
+                                 f"which does not run before it")
+        self.loaded_dtype: Optional[str] = None
+
+    def parts(self) -> List[Part]:
+        out = []
+        for top in [self.embedding] + self.blocks + [self.final_norm, self.head]:
+            out.extend(walk(top))
+        return out
+
+    def tensor_reqs(self) -> List[TensorReq]:
+        reqs = []
+        for p in self.parts():
+            reqs.extend(p.tensor_reqs())
+        return reqs
+
+    def load(self, weights, rt, dtype: str) -> None:
+        for p in self.parts():
+            p.load(weights, rt, dtype)
+        self.loaded_dtype = dtype
+
+    def cache_needs(self) -> List[object]:
+        """Per entry of the order: what its mixer keeps (None for an entry that
+        reads another entry's cache, or keeps nothing)."""
+        out = []
+        for call in self.plan.order:
+            if call.cache_of is not None:
+                out.append(None)
+            else:
+                out.append(self.blocks[call.layer].mixer.cache_need())
+        return out
+
+    def forward(self, ctx, caches: List[CallCache], logit_rows, n_rows: int, logits: Tensor):
+        """Run the step's tokens through every entry of the order; write float
+        logits of the rows ``logit_rows`` (device int32 pointer) into ``logits``."""
+        h = self.embedding.forward(ctx)
+        for i, call in enumerate(self.plan.order):
+            cache = caches[call.cache_of if call.cache_of is not None else i]
+            self.blocks[call.layer].forward(ctx, h, cache)
+        if n_rows:
+            x = self.final_norm.forward(ctx, h, out_rows=(logit_rows, n_rows))
+            self.head.forward(ctx, x, logits)
+        return logits

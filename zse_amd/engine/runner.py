@@ -1,0 +1,334 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+``StepRunner.step(entries)`` takes, for each request, the tokens that follow
+what it already has in the cache: a portion of a prompt of any length beside
+single decoded tokens, cut anywhere.  All entries run as one batch: tokens are
+laid out flat, each with its position, its request and, per cache group, the
+place in the pages where its key and value go; attention then reads the cache
+alone.  Logits come back for the places that were asked for.
+
+The reference has three disjoint calls instead (a whole new prompt, M
+sequences of one token, K tokens of one sequence: orchestrator/model_runner.py:290,
+843, 761), rebuilds and uploads tokens, positions, packed block tables and
+lengths for each (model_runner.py:873-884), and cannot continue a prompt
+(cache/page_table.py:58-59).  Decode steps of a fixed shape are captured into a
+HIP graph per batch size as there (model_runner.py:1806-1932).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from ..cache.manager import CacheManager, GroupInfo, group_needs
+from ..cache.pages import OutOfPages
+from ..parts.base import PagedKV, StateNeed
+from ..runtime.device import BF16, F32, I32, ITEMSIZE, Runtime, Tensor, canonical_dtype
+from .model import CallCache, Model
+
+
+@dataclass
+class StepEntry:
+    req: object                      # request id
+    tokens: Sequence[int]            # its next tokens
+    want: Sequence[int] = ()         # places among these tokens whose logits are wanted
+
+
+@dataclass
+class GroupView:
+    block_table: int                 # device pointer, int32 [R, max_blocks]
+    max_blocks: int
+    slot_map: int                    # device pointer, int32 [T]
+    page_size: int
+
+
+class Arena:
+    """Bump allocator over device memory for a step's activations.  It grows by
+    whole chunks when a step needs more and keeps them; ``mark``/``release``
+    give a layer's buffers back for the next layer."""
+
+    ALIGN = 256
+
+    def __init__(self, rt: Runtime, chunk_bytes: int = 64 << 20):
+        self.rt = rt
+        self.chunk_bytes = chunk_bytes
+        self.chunks: List[Tensor] = []
+        self.cur = 0          # chunk index
+        self.off = 0
+        self.frozen = False   # no growth while a graph is being captured
+
+    def reset(self):
+        self.cur, self.off = 0, 0
+
+    def mark(self):
+        return (self.cur, self.off)
+
+    def release(self, m):
+        self.cur, self.off = m
+
+    def alloc(self, shape, dtype: str) -> Tensor:
+        n = ITEMSIZE[dtype]
+        for s in shape:
+            n *= int(s)
+        n = (max(n, 1) + self.ALIGN - 1) // self.ALIGN * self.ALIGN
+        while True:
+            if self.cur < len(self.chunks) and self.off + n <= self.chunks[self.cur].nbytes:
+                t = Tensor(self.chunks[self.cur].ptr + self.off, shape, dtype, self.chunks[self.cur].owner)
+                self.off += n
+                return t
+            if self.cur + 1 < len(self.chunks):
+                self.cur += 1
+                self.off = 0
+                continue
+            if self.frozen:
+                raise RuntimeError("activation arena would grow during graph capture")
+            self.chunks.append(self._new_chunk(max(n, self.chunk_bytes)))
+            self.cur = len(self.chunks) - 1
+            self.off = 0
+
+    def _new_chunk(self, nbytes: int) -> Tensor:
+        return self.rt.empty(((nbytes + 3) // 4,), F32)
+
+
+class StepContext:
+    """What parts see of a step."""
+
+    def __init__(self, runner: "StepRunner"):
+        self.runner = runner
+        self.rt = runner.rt
+        self.k = runner.k
+        self.dtype = runner.dtype
+        self.tuned = runner.tuned
+        self.stream = runner.rt.stream
+        self.arena = runner.arena
+        self.workspace = runner.workspace
+        self.T = 0
+        self.R = 0
+        self.tokens = self.positions = self.req_of_token = self.q_start = self.ctx_len = 0
+        self.slot_of_req = 0
+        self.groups: List[GroupView] = []
+        self.max_q_len = 0
+        self.max_ctx = 0
+        self.entries: List[Tuple[object, int, int, int]] = []   # (req, slot, start, n) on the host
+        self.state = None            # Tensor uint8-as-float32 words [max_seqs, slot_words] or None
+        self.slot_bytes = 0
+
+    def alloc(self, shape, dtype: Optional[str] = None) -> Tensor:
+        return self.arena.alloc(shape, dtype or self.dtype)
+
+    def group(self, gid: int) -> GroupView:
+        return self.groups[gid]
+
+
+class StepRunner:
+    def __init__(self, model: Model, rt: Runtime, dtype: str, page_size: int = 16,
+                 num_pages: Optional[int] = None, cache_tokens: Optional[int] = None,
+                 max_seqs: int = 64, max_batch_tokens: int = 4096, max_model_len: Optional[int] = None,
+                 tuned: bool = True, use_graphs: bool = True):
+        self.model, self.rt = model, rt
+        self.dtype = canonical_dtype(dtype)
+        if model.loaded_dtype != self.dtype:
+            raise ValueError(f"the model's weights are {model.loaded_dtype}, the runner wants {self.dtype}")
+        self.k = rt.kernels(self.dtype)
+        self.tuned = bool(tuned)
+        self.use_graphs = bool(use_graphs) and self.tuned
+        self.page_size = int(page_size)
+        self.max_seqs = int(max_seqs)
+        self.max_batch_tokens = int(max_batch_tokens)
+        self.max_model_len = int(max_model_len or model.plan.max_position)
+        self.vocab = model.plan.vocab_size
+
+        # ---- cache layout
+        needs = model.cache_needs()
+        groups = group_needs(needs)
+        if num_pages is None:
+            tokens = cache_tokens if cache_tokens is not None else self.max_model_len
+            num_pages = -(-int(tokens) // self.page_size)
+        for g in groups:
+            g.num_pages = int(num_pages)
+        slot_bytes = 0
+        self.caches: List[CallCache] = []
+        gid_of = {}
+        for gid, g in enumerate(groups):
+            for c in g.calls:
+                gid_of[c] = gid
+        item = ITEMSIZE[self.dtype]
+        for i, need in enumerate(needs):
+            cc = CallCache(need=need)
+            if isinstance(need, PagedKV):
+                cc.group = gid_of[i]
+                shape = (num_pages, need.num_kv_heads, self.page_size, need.head_dim)
+                cc.k = rt.zeros(shape, self.dtype)
+                cc.v = rt.zeros(shape, self.dtype)
+            elif isinstance(need, StateNeed):
+                cc.state_offset = slot_bytes
+                cc.state_bytes = int(need.nbytes)
+                slot_bytes += (int(need.nbytes) + 15) // 16 * 16
+            self.caches.append(cc)
+        self.slot_bytes = slot_bytes
+        self.manager = CacheManager(groups, self.page_size, self.max_seqs, self.max_model_len, slot_bytes)
+        self.state = rt.zeros((self.max_seqs, max(slot_bytes // 4, 1)), F32) if slot_bytes else None
+
+        # ---- step buffers
+        self.arena = Arena(rt)
+        self.workspace = rt.zeros((self._workspace_words(),), F32)
+        G = len(groups)
+        self.max_blocks = self.manager.max_blocks
+        cap = self._meta_words(self.max_batch_tokens, self.max_seqs, G)
+        self.meta_host = rt.pinned(cap * 4)
+        self.meta_dev = rt.empty((cap,), I32)
+        self.meta_copied = rt.event()
+        rt.record(self.meta_copied)
+        self.logits: Optional[Tensor] = None
+        self.graphs: Dict[int, dict] = {}
+        self.steps_run = 0
+
+    # ------------------------------------------------------------------ sizes
+    def _workspace_words(self) -> int:
+        # partial results of split attention: sized by the bf16 kernels' own need
+        return 1 << 20 if self.dtype == F32 else (32 << 20)
+
+    def _meta_words(self, T: int, R: int, G: int) -> int:
+        return 4 * T + (R + 1) + 2 * R + G * (T + R * self.max_blocks) + 64
+
+    def cache_bytes(self) -> int:
+        return sum(c.k.nbytes + c.v.nbytes for c in self.caches if c.k is not None)
+
+    # ------------------------------------------------------------------ requests
+    def add(self, req) -> int:
+        slot = self.manager.add(req)
+        if self.state is not None:
+            self.rt.zero_(self.state.rows(slot, slot + 1))
+        return slot
+
+    def finish(self, req) -> None:
+        self.manager.release(req)
+
+    # ------------------------------------------------------------------ the step
+    def _pack(self, entries: Sequence[StepEntry], T_pad: int, R_pad: int):
+        """Fill the pinned host buffer; returns offsets (in words) and counts."""
+        m, ps = self.manager, self.page_size
+        G = len(m.groups)
+        T = sum(len(e.tokens) for e in entries)
+        R = len(entries)
+        off = {}
+        cur = 0
+
+        def take(name, n):
+            nonlocal cur
+            off[name] = cur
+            cur += n
+            return self.meta_host.array(off[name] * 4, n, np.int32)
+
+        tokens = take("tokens", T_pad)
+        positions = take("positions", T_pad)
+        req_of_token = take("req_of_token", T_pad)
+        logit_rows = take("logit_rows", T_pad)
+        q_start = take("q_start", R_pad + 1)
+        ctx_len = take("ctx_len", R_pad)
+        slot_of_req = take("slot_of_req", R_pad)
+        slot_maps = [take(f"slot_map{g}", T_pad) for g in range(G)]
+        tables = [take(f"table{g}", R_pad * self.max_blocks).reshape(R_pad, self.max_blocks)
+                  for g in range(G)]
+        tokens[T:] = 0
+        positions[T:] = -1
+        req_of_token[T:] = 0
+        for sm in slot_maps:
+            sm[T:] = -1
+        t = 0
+        n_rows = 0
+        host_entries = []
+        max_q = max_ctx = 0
+        for r, e in enumerate(entries):
+            n = len(e.tokens)
+            start = m.computed(e.req)
+            tokens[t:t + n] = np.asarray(e.tokens, dtype=np.int32)
+            positions[t:t + n] = np.arange(start, start + n, dtype=np.int32)
+            req_of_token[t:t + n] = r
+            q_start[r] = t
+            ctx_len[r] = start + n
+            slot_of_req[r] = m.slot(e.req)
+            for g in range(G):
+                slot_maps[g][t:t + n] = m.slot_mapping(e.req, g, start, n)
+                m.fill_table_row(e.req, g, tables[g][r])
+            for w in e.want:
+                if not (0 <= w < n):
+                    raise ValueError(f"request {e.req!r}: wanted place {w} is not among its {n} tokens")
+                logit_rows[n_rows] = t + w
+                n_rows += 1
+            host_entries.append((e.req, m.slot(e.req), start, n))
+            max_q, max_ctx = max(max_q, n), max(max_ctx, start + n)
+            t += n
+        q_start[R:] = T
+        ctx_len[R:] = 0
+        slot_of_req[R:] = 0
+        for g in range(G):
+            tables[g][R:] = -1
+        return off, cur, T, R, n_rows, host_entries, max_q, max_ctx
+
+    def _context(self, off, T_pad, R_pad, host_entries, max_q, max_ctx) -> StepContext:
+        ctx = StepContext(self)
+        base = self.meta_dev.ptr
+        p = lambda name: base + off[name] * 4
+        ctx.T, ctx.R = T_pad, R_pad
+        ctx.tokens, ctx.positions, ctx.req_of_token = p("tokens"), p("positions"), p("req_of_token")
+        ctx.q_start, ctx.ctx_len, ctx.slot_of_req = p("q_start"), p("ctx_len"), p("slot_of_req")
+        ctx.logit_rows = p("logit_rows")
+        ctx.groups = [GroupView(p(f"table{g}"), self.max_blocks, p(f"slot_map{g}"), self.page_size)
+                      for g in range(len(self.manager.groups))]
+        ctx.entries = host_entries
+        ctx.max_q_len, ctx.max_ctx = max_q, max_ctx
+        ctx.state, ctx.slot_bytes = self.state, self.slot_bytes
+        return ctx
+
+    def _ensure_logits(self, rows: int):
+        if self.logits is None or self.logits.shape[0] < rows:
+            self.rt.sync()
+            self.logits = None
+            self.logits = self.rt.empty((max(rows, 8), self.vocab), F32)
+
+    def step(self, entries: Sequence[StepEntry], download: bool = True):
+        """Run one step.  Returns float32 logits [wanted, vocab] on the host
+        (``download=False``: the device tensor, valid until the next step)."""
+        entries = [e for e in entries if len(e.tokens) > 0]
+        if not entries:
+            return np.zeros((0, self.vocab), np.float32) if download else None
+        m = self.manager
+        seen = set()
+        for e in entries:
+            if e.req in seen:
+                raise ValueError(f"request {e.req!r} appears twice in one step")
+            seen.add(e.req)
+            for tok in e.tokens:
+                if not (0 <= int(tok) < self.vocab):
+                    raise ValueError(f"request {e.req!r}: token id {tok} is outside the vocabulary "
+                                     f"of {self.vocab}")
+        T = sum(len(e.tokens) for e in entries)
+        R = len(entries)
+        if T > self.max_batch_tokens or R > self.max_seqs:
+            raise ValueError(f"step of {T} tokens in {R} requests exceeds the limits "
+                             f"({self.max_batch_tokens} tokens, {self.max_seqs} requests)")
+        for e in entries:
+            if not m.has(e.req):
+                self.add(e.req)
+        for e in entries:
+            upto = m.computed(e.req) + len(e.tokens)
+            if not m.reserve(e.req, upto):
+                raise OutOfPages(f"request {e.req!r} needs pages for {upto} tokens and the pool "
+                                 f"cannot give them: {m.stats()}")
+        self.rt.wait_event(self.meta_copied)     # the last step's copy has left the host buffer
+        off, words, T, R, n_rows, host_entries, max_q, max_ctx = self._pack(entries, T, R)
+        self._ensure_logits(n_rows)
+        self.rt.copy_h2d_async(self.meta_dev.ptr, self.meta_host.ptr, words * 4)
+        self.rt.record(self.meta_copied)
+        ctx = self._context(off, T, R, host_entries, max_q, max_ctx)
+        self.arena.reset()
+        self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, self.logits.rows(0, n_rows))
+        for e in entries:
+            m.commit(e.req, m.computed(e.req) + len(e.tokens))
+        self.steps_run += 1
+        out = self.logits.rows(0, n_rows)
+        if not download:
+            return out
+        return self.rt.download(out)

@@ -1,0 +1,4 @@
+"""Parts a model is put together from.  Importing the package registers the built-in kinds."""
+from . import attention, block, embedding, ffn, norm, position  # noqa: F401
+from .base import (PagedKV, Part, StateNeed, TensorReq, build_part, register_part,
+                   unregister_part, walk)

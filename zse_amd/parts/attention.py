@@ -1,0 +1,88 @@
+"""Grouped-query softmax attention over the paged cache.
+
+One forward for every kind of step: project q, k, v in one product, rotate q
+and k and store k, v at each token's place in the cache, then let every token
+attend to the cache alone, over the positions [max(0, pos - window + 1), pos]
+(all earlier positions without a window).  The reference writes the cache
+first as well (orchestrator/model_runner.py:1184-1194) but its prefill reads
+contiguous K/V and never masks a window (orchestrator/kernels.py:883,
+model_runner.py:489-490); its scale is fixed at 1/sqrt(head_dim)
+(model_runner.py:80) where this part takes the scale and the soft cap as
+parameters.  q, k, v stay separate products in the reference
+(model_runner.py:1151-1165); here they are one.
+"""
+from __future__ import annotations
+
+from typing import List
+
+from ..runtime.device import BF16, Tensor
+from .base import PagedKV, Part, TensorReq, build_part, register_part
+from .ops import linear
+
+
+class PagedAttention(Part):
+    def __init__(self, spec):
+        s = self.spec = spec
+        if s.num_heads % s.num_kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        if s.head_dim % 16 or s.head_dim > 256:
+            raise ValueError(f"head_dim must be a multiple of 16 up to 256, got {s.head_dim}")
+        self.position = build_part("position", s.position)
+        self.shared_kv = "k" not in s.names        # reads another call's cache, writes none
+        self.w_qkv = self.w_o = None
+
+    def children(self):
+        return [self.position]
+
+    def tensor_reqs(self) -> List[TensorReq]:
+        s = self.spec
+        q = TensorReq(s.names["q"], (s.num_heads * s.head_dim, s.hidden_size))
+        o = TensorReq(s.names["o"], (s.hidden_size, s.num_heads * s.head_dim))
+        if self.shared_kv:
+            return [q, o]
+        kv = (s.num_kv_heads * s.head_dim, s.hidden_size)
+        return [q, TensorReq(s.names["k"], kv), TensorReq(s.names["v"], kv), o]
+
+    def load(self, weights, rt, dtype):
+        s = self.spec
+        names = [s.names["q"]] if self.shared_kv else [s.names[r] for r in ("q", "k", "v")]
+        self.w_qkv = weights.matrix(names)
+        self.w_o = weights.matrix([s.names["o"]])
+
+    def cache_need(self):
+        s = self.spec
+        return PagedKV(s.num_kv_heads, s.head_dim, s.window)
+
+    def forward(self, ctx, x: Tensor, cache) -> Tensor:
+        s, k = self.spec, ctx.k
+        T = x.shape[0]
+        nh, nkv, hd = s.num_heads, s.num_kv_heads, s.head_dim
+        n_store = 0 if self.shared_kv else nkv
+        width = (nh + 2 * n_store) * hd
+        qkv = linear(ctx, x, self.w_qkv, ctx.alloc((T, width)))
+        g = ctx.group(cache.group)
+        tables = self.position.rotary_tables()
+        if tables is None:
+            self.position.apply(ctx, qkv, nh, n_store, hd)
+            inv_freq, rotary_dim = 0, 0
+        else:
+            inv_freq, rotary_dim = tables[0].ptr, tables[1]
+        k.zk_rope_cache_write(qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map,
+                              inv_freq or None, rotary_dim, cache.k.ptr, cache.v.ptr, T, nh, n_store,
+                              hd, g.page_size, ctx.stream)
+        o = ctx.alloc((T, nh * hd))
+        cap = float(s.softcap) if s.softcap else 0.0
+        win = int(s.window) if s.window else 0
+        if ctx.dtype == BF16 and ctx.tuned and k.has("zk_attention_bf16"):
+            k.zk_attention_bf16(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
+                                ctx.req_of_token, ctx.positions, ctx.q_start, ctx.R, o.ptr, T, nh,
+                                nkv, hd, g.page_size, s.scale, cap, win, ctx.max_q_len, ctx.max_ctx,
+                                ctx.workspace.ptr, ctx.workspace.nbytes, ctx.stream)
+        else:
+            k.zk_attention_plain(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table,
+                                 g.max_blocks, ctx.req_of_token, ctx.positions, o.ptr, T, nh, nkv,
+                                 hd, g.page_size, s.scale, cap, win, ctx.stream)
+        return linear(ctx, o, self.w_o, ctx.alloc((T, s.hidden_size)))
+
+
+register_part("mixer", "attention", PagedAttention)

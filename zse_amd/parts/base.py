@@ -1,0 +1,92 @@
+"""What every part is: a description-driven object with tensors and a forward.
+
+A part is built from its spec alone (no device needed), says which checkpoint
+tensors it wants (``tensor_reqs``), later binds them on the device (``load``)
+and runs on the tokens of a step (``forward``).  No part knows which model it
+belongs to.  Kinds are looked up in the registries below; a new kind is added
+with ``register_part`` from anywhere, tests included.
+
+Interfaces, by slot:
+
+  norm      forward(ctx, x, out_rows=None) -> Tensor[rows, size] activations.
+            ``x`` is the float residual stream or an activation tensor;
+            ``out_rows`` (device int32 pointer, count) picks rows.
+  position  rotary_tables() -> (inv_freq Tensor float32 [rotary_dim/2], rotary_dim)
+            or None; apply(ctx, qkv, num_heads, num_kv_heads, head_dim) for an
+            encoding that is not a rotation by position.
+  mixer     cache_need() -> PagedKV | StateNeed | None;
+            forward(ctx, x, cache) -> Tensor[T, hidden]
+  ffn       forward(ctx, x) -> Tensor[T, hidden]
+  block     forward(ctx, h, cache): updates the float stream ``h`` in place.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional, Tuple
+
+ROLE_MATRIX = "matrix"   # used in matrix products: stored in the compute dtype
+ROLE_GAIN = "gain"       # norm gains and other vectors: kept as float32
+
+
+@dataclass(frozen=True)
+class TensorReq:
+    name: str
+    shape: Tuple[int, ...]
+    role: str = ROLE_MATRIX
+    init_std: Optional[float] = None    # random-weights mode: None = the mode's default for the role
+
+
+@dataclass(frozen=True)
+class PagedKV:
+    """The mixer keeps keys and values per token, in pages.  ``window``: only the
+    last ``window`` positions are ever read again (None: all of them)."""
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int]
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """The mixer keeps ``nbytes`` of state per request, whatever its length."""
+    nbytes: int
+
+
+class Part:
+    spec = None
+
+    def tensor_reqs(self) -> List[TensorReq]:
+        return []
+
+    def load(self, weights, rt, dtype: str) -> None:
+        """Bind device tensors from a weight source (see zse_amd.weights.loader)."""
+
+    def children(self) -> List["Part"]:
+        return []
+
+
+_REGISTRIES: Dict[str, Dict[str, Callable]] = {
+    "norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}, "embedding": {}, "head": {},
+}
+
+
+def register_part(slot: str, kind: str, factory: Callable) -> None:
+    """``factory(spec) -> Part``."""
+    _REGISTRIES[slot][kind] = factory
+
+
+def unregister_part(slot: str, kind: str) -> None:
+    _REGISTRIES[slot].pop(kind, None)
+
+
+def build_part(slot: str, spec) -> Part:
+    reg = _REGISTRIES[slot]
+    kind = getattr(spec, "kind", None)
+    if kind not in reg:
+        raise KeyError(f"no {slot} part of kind {kind!r}; registered: {sorted(reg)}")
+    return reg[kind](spec)
+
+
+def walk(part: Part):
+    yield part
+    for c in part.children():
+        yield from walk(c)

@@ -1,0 +1,69 @@
+"""Token embedding into the float stream, and the output head.
+
+The gather writes float rows (orchestrator/kernels.py:1789-1806) times a scale,
+sqrt(hidden) for Gemma (orchestrator/model_runner.py:153-158, 332-339).  The head
+multiplies by the embedding matrix itself when the weights are tied
+(model_runner.py:566-572) and soft-caps the float logits (kernels.py:1714-1727,
+model_runner.py:573-576); only the rows that were asked for are computed, where
+the reference computes all of them (model_runner.py:362-373).
+"""
+from __future__ import annotations
+
+from typing import List
+
+import numpy as np
+
+from ..runtime.device import BF16, F32, Tensor
+from .base import Part, TensorReq, register_part
+from .ops import linear
+
+
+class Embedding(Part):
+    def __init__(self, spec):
+        self.spec = spec
+        self.table = None
+        self.scale = float(spec.scale)
+
+    def tensor_reqs(self) -> List[TensorReq]:
+        return [TensorReq(self.spec.weight, (self.spec.vocab_size, self.spec.hidden_size))]
+
+    def load(self, weights, rt, dtype):
+        self.table = weights.matrix([self.spec.weight])
+        # the scalar is kept in the table's storage type, as the reference keeps its own
+        # (model_runner.py:155-158); the product is float
+        s = np.float32(self.spec.scale)
+        if dtype == BF16:
+            from ..weights.safetensors import bf16_bits_to_f32, f32_to_bf16_bits
+            s = bf16_bits_to_f32(f32_to_bf16_bits(np.array([s])))[0]
+        self.scale = float(s)
+
+    def forward(self, ctx) -> Tensor:
+        s = self.spec
+        h = ctx.alloc((ctx.T, s.hidden_size), F32)
+        ctx.k.zk_embed(self.table.ptr, ctx.tokens, h.ptr, self.scale, ctx.T, s.hidden_size,
+                       s.vocab_size, ctx.stream)
+        return h
+
+
+class LMHead(Part):
+    def __init__(self, spec):
+        self.spec = spec
+        self.weight = None
+
+    def tensor_reqs(self) -> List[TensorReq]:
+        return [TensorReq(self.spec.weight, (self.spec.vocab_size, self.spec.hidden_size))]
+
+    def load(self, weights, rt, dtype):
+        self.weight = weights.matrix([self.spec.weight])
+
+    def forward(self, ctx, x: Tensor, out: Tensor) -> Tensor:
+        """x: normed rows [K, hidden]; out: float logits [K, vocab]."""
+        s = self.spec
+        linear(ctx, x, self.weight, out)
+        if s.softcap:
+            ctx.k.zk_softcap(out.ptr, out.numel, float(s.softcap), ctx.stream)
+        return out
+
+
+register_part("embedding", "embedding", Embedding)
+register_part("head", "lm_head", LMHead)

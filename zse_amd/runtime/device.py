@@ -1,0 +1,366 @@
+"""The device side seen from Python: memory, streams, events, graphs, kernels.
+
+Everything goes through ctypes into the libraries built from ``zse_amd/csrc``,
+in the manner of the reference's ``GPUMemory`` and ``KernelLauncher``
+(zse-compiler/zse_compiler/runtime/memory.py:71-447, launcher.py:72-175).  There
+is no fallback: without a GPU or without the libraries, ``Runtime()`` raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Dict, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import build
+
+F32 = "float32"
+BF16 = "bfloat16"
+I32 = "int32"
+F64 = "float64"
+ITEMSIZE = {F32: 4, BF16: 2, I32: 4, F64: 8}
+NUMPY_OF = {F32: np.float32, BF16: np.uint16, I32: np.int32, F64: np.float64}
+DTYPE_ALIASES = {"float32": F32, "fp32": F32, "f32": F32, "bfloat16": BF16, "bf16": BF16}
+
+
+def canonical_dtype(name: str) -> str:
+    try:
+        return DTYPE_ALIASES[str(name).lower()]
+    except KeyError:
+        raise ValueError(f"dtype must be one of {sorted(DTYPE_ALIASES)}, got {name!r}") from None
+
+
+class DeviceError(RuntimeError):
+    pass
+
+
+class Tensor:
+    """A view of device memory: pointer, shape, dtype.  Row-major, contiguous."""
+
+    __slots__ = ("ptr", "shape", "dtype", "owner")
+
+    def __init__(self, ptr: int, shape: Sequence[int], dtype: str, owner=None):
+        self.ptr = int(ptr)
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = dtype
+        self.owner = owner      # keeps the allocation alive
+
+    @property
+    def numel(self) -> int:
+        n = 1
+        for s in self.shape:
+            n *= s
+        return n
+
+    @property
+    def nbytes(self) -> int:
+        return self.numel * ITEMSIZE[self.dtype]
+
+    def view(self, *shape) -> "Tensor":
+        t = Tensor(self.ptr, shape, self.dtype, self.owner)
+        if t.numel != self.numel:
+            raise ValueError(f"cannot view {self.shape} as {shape}")
+        return t
+
+    def rows(self, begin: int, end: int) -> "Tensor":
+        """Rows [begin, end) of the first axis."""
+        if not (0 <= begin <= end <= self.shape[0]):
+            raise IndexError(f"rows {begin}:{end} of {self.shape}")
+        inner = self.numel // self.shape[0] if self.shape[0] else 0
+        return Tensor(self.ptr + begin * inner * ITEMSIZE[self.dtype],
+                      (end - begin,) + self.shape[1:], self.dtype, self.owner)
+
+    def __repr__(self):
+        return f"Tensor({self.dtype}, {self.shape}, 0x{self.ptr:x})"
+
+
+class Allocation:
+    """Owns one device allocation; freed when dropped or closed."""
+
+    def __init__(self, rt: "Runtime", nbytes: int):
+        self.rt = rt
+        self.nbytes = int(nbytes)
+        p = C.c_void_p()
+        rt._check(rt.lib.zrt_malloc(C.byref(p), C.c_size_t(max(self.nbytes, 4))), "malloc")
+        self.ptr = p.value
+        rt.allocated += self.nbytes
+
+    def close(self):
+        if self.ptr:
+            self.rt.lib.zrt_free(C.c_void_p(self.ptr))
+            self.rt.allocated -= self.nbytes
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class PinnedBuffer:
+    """Page-locked host memory, seen as a numpy byte array."""
+
+    def __init__(self, rt: "Runtime", nbytes: int):
+        self.rt = rt
+        self.nbytes = int(nbytes)
+        p = C.c_void_p()
+        rt._check(rt.lib.zrt_host_alloc(C.byref(p), C.c_size_t(max(self.nbytes, 8))), "host alloc")
+        self.ptr = p.value
+        self.bytes = np.ctypeslib.as_array((C.c_uint8 * max(self.nbytes, 8)).from_address(self.ptr))
+
+    def array(self, offset: int, count: int, dtype) -> np.ndarray:
+        dt = np.dtype(dtype)
+        return self.bytes[offset:offset + count * dt.itemsize].view(dt)
+
+    def close(self):
+        if self.ptr:
+            self.bytes = None
+            self.rt.lib.zrt_host_free(C.c_void_p(self.ptr))
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+@dataclass
+class DeviceInfo:
+    name: str
+    arch: str
+    total_memory: int
+    free_memory: int
+    compute_units: int
+
+
+_VP, _I, _F, _SZ, _U64 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint64
+
+# name -> argument types (all return int; 0 = success)
+KERNEL_SIGNATURES = {
+    "zk_embed": [_VP, _VP, _VP, _F, _I, _I, _I, _VP],
+    "zk_rmsnorm": [_VP, _I, _VP, _VP, _VP, _F, _I, _I, _I, _VP],
+    "zk_norm_add_norm": [_VP, _VP, _F, _I, _VP, _VP, _F, _I, _VP, _I, _I, _VP],
+    "zk_gated_act": [_VP, _VP, _I, _I, _I, _VP],
+    "zk_softcap": [_VP, _SZ, _F, _VP],
+    "zk_rope_cache_write": [_VP, _VP, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "zk_convert": [_VP, _I, _VP, _I, _SZ, _VP],
+    "zk_fill_normal": [_VP, _I, _SZ, _U64, _U64, _F, _F, _VP],
+    "zk_zero": [_VP, _SZ, _VP],
+    "zk_gemm_plain": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "zk_attention_plain": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _F,
+                           _I, _VP],
+    "zk_argmax": [_VP, _VP, _I, _I, _VP],
+    "zk_sample": [_VP, _VP, _VP, _VP, _VP, _I, _I, _VP],
+}
+# present only in the bf16 library
+BF16_KERNEL_SIGNATURES = {}
+
+
+class KernelLibrary:
+    """One built kernel library; calling ``lib.zk_x(...)`` raises on a non-zero status."""
+
+    def __init__(self, path: str, dtype: str):
+        self.path = path
+        self.dtype = dtype
+        self._dll = C.CDLL(path)
+        self._dll.zk_last_error.restype = C.c_char_p
+        sigs = dict(KERNEL_SIGNATURES)
+        if dtype == BF16:
+            sigs.update(BF16_KERNEL_SIGNATURES)
+        for name, args in sigs.items():
+            try:
+                fn = getattr(self._dll, name)
+            except AttributeError:
+                raise DeviceError(f"{path} lacks {name}: rebuild with `python -m zse_amd build`") from None
+            fn.argtypes = args
+            fn.restype = C.c_int
+            setattr(self, name, self._wrap(name, fn))
+        want = 1 if dtype == BF16 else 0
+        if self._dll.zk_act_is_bf16() != want:
+            raise DeviceError(f"{path} was built for the other storage type")
+
+    def has(self, name: str) -> bool:
+        return hasattr(self, name)
+
+    def _wrap(self, name, fn):
+        dll = self._dll
+
+        def call(*a):
+            rc = fn(*a)
+            if rc != 0:
+                raise DeviceError(f"{name} failed ({rc}): {dll.zk_last_error().decode()}")
+        call.__name__ = name
+        return call
+
+
+class Runtime:
+    """The process's handle on GPU 0 (or ``device``)."""
+
+    _instance: Optional["Runtime"] = None
+
+    @classmethod
+    def get(cls, device: int = 0) -> "Runtime":
+        if cls._instance is None:
+            cls._instance = Runtime(device)
+        return cls._instance
+
+    def __init__(self, device: int = 0):
+        path = build.ensure("runtime")
+        self.lib = C.CDLL(path)
+        self.lib.zrt_last_error.restype = C.c_char_p
+        for name in ("zrt_malloc", "zrt_free", "zrt_host_alloc", "zrt_host_free", "zrt_h2d", "zrt_d2h",
+                     "zrt_d2d", "zrt_stream_create", "zrt_stream_destroy", "zrt_stream_sync",
+                     "zrt_device_sync", "zrt_event_create", "zrt_event_record", "zrt_event_sync",
+                     "zrt_event_elapsed_ms", "zrt_event_destroy", "zrt_capture_begin",
+                     "zrt_capture_end", "zrt_graph_launch", "zrt_graph_destroy", "zrt_init",
+                     "zrt_device_count", "zrt_device_info"):
+            getattr(self.lib, name).restype = C.c_int
+        self.lib.zrt_h2d.argtypes = [_VP, _VP, _SZ, _VP, _I]
+        self.lib.zrt_d2h.argtypes = [_VP, _VP, _SZ, _VP, _I]
+        self.lib.zrt_d2d.argtypes = [_VP, _VP, _SZ, _VP]
+        self.lib.zrt_free.argtypes = [_VP]
+        self.lib.zrt_host_free.argtypes = [_VP]
+        self.lib.zrt_stream_sync.argtypes = [_VP]
+        self.lib.zrt_stream_destroy.argtypes = [_VP]
+        self.lib.zrt_event_record.argtypes = [_VP, _VP]
+        self.lib.zrt_event_sync.argtypes = [_VP]
+        self.lib.zrt_event_elapsed_ms.argtypes = [_VP, _VP, _VP]
+        self.lib.zrt_event_destroy.argtypes = [_VP]
+        self.lib.zrt_capture_begin.argtypes = [_VP]
+        self.lib.zrt_capture_end.argtypes = [_VP, _VP]
+        self.lib.zrt_graph_launch.argtypes = [_VP, _VP]
+        self.lib.zrt_graph_destroy.argtypes = [_VP]
+        n = C.c_int(0)
+        rc = self.lib.zrt_device_count(C.byref(n))
+        if rc != 0 or n.value < 1:
+            raise DeviceError("no HIP device is visible: this engine runs on a GPU only "
+                              f"({self.lib.zrt_last_error().decode()})")
+        self.device = device
+        self._check(self.lib.zrt_init(C.c_int(device)), "init")
+        self.allocated = 0
+        self._kernels: Dict[str, KernelLibrary] = {}
+        s = C.c_void_p()
+        self._check(self.lib.zrt_stream_create(C.byref(s)), "stream create")
+        self.stream = s.value
+
+    # -- errors
+    def _check(self, rc: int, what: str):
+        if rc != 0:
+            raise DeviceError(f"{what} failed ({rc}): {self.lib.zrt_last_error().decode()}")
+
+    # -- info
+    def info(self) -> DeviceInfo:
+        name = C.create_string_buffer(256)
+        arch = C.create_string_buffer(256)
+        total, free = C.c_size_t(), C.c_size_t()
+        cus = C.c_int()
+        self._check(self.lib.zrt_device_info(C.c_int(self.device), name, 256, C.byref(total),
+                                             C.byref(free), C.byref(cus), arch, 256), "device info")
+        return DeviceInfo(name.value.decode(), arch.value.decode(), total.value, free.value, cus.value)
+
+    # -- kernels
+    def kernels(self, dtype: str) -> KernelLibrary:
+        dtype = canonical_dtype(dtype)
+        if dtype not in self._kernels:
+            name = "kernels_bf16" if dtype == BF16 else "kernels_f32"
+            self._kernels[dtype] = KernelLibrary(build.ensure(name), dtype)
+        return self._kernels[dtype]
+
+    # -- memory
+    def empty(self, shape, dtype: str) -> Tensor:
+        shape = tuple(int(s) for s in (shape if isinstance(shape, (tuple, list)) else (shape,)))
+        n = ITEMSIZE[dtype]
+        for s in shape:
+            n *= s
+        a = Allocation(self, n)
+        return Tensor(a.ptr, shape, dtype, a)
+
+    def zeros(self, shape, dtype: str) -> Tensor:
+        t = self.empty(shape, dtype)
+        self.zero_(t)
+        return t
+
+    def zero_(self, t: Tensor):
+        nbytes = (t.nbytes + 3) // 4 * 4
+        self.kernels(F32).zk_zero(t.ptr, nbytes, self.stream)
+
+    def pinned(self, nbytes: int) -> PinnedBuffer:
+        return PinnedBuffer(self, nbytes)
+
+    def upload(self, arr: np.ndarray, dtype: Optional[str] = None) -> Tensor:
+        """Copy a host array to a new device tensor (synchronous).  ``dtype`` only
+        labels the result; the bytes go up as they are."""
+        arr = np.ascontiguousarray(arr)
+        if dtype is None:
+            dtype = {np.dtype(np.float32): F32, np.dtype(np.int32): I32, np.dtype(np.uint16): BF16,
+                     np.dtype(np.float64): F64}[arr.dtype]
+        t = self.empty(arr.shape, dtype)
+        if t.nbytes != arr.nbytes:
+            raise ValueError(f"{arr.dtype} array does not store {dtype}")
+        self.copy_h2d(t.ptr, arr)
+        return t
+
+    def copy_h2d(self, dst_ptr: int, arr: np.ndarray):
+        arr = np.ascontiguousarray(arr)
+        if arr.nbytes:
+            self._check(self.lib.zrt_h2d(dst_ptr, arr.ctypes.data, arr.nbytes, self.stream, 0), "h2d")
+
+    def copy_h2d_async(self, dst_ptr: int, host_ptr: int, nbytes: int):
+        if nbytes:
+            self._check(self.lib.zrt_h2d(dst_ptr, host_ptr, nbytes, self.stream, 1), "h2d")
+
+    def copy_d2d(self, dst_ptr: int, src_ptr: int, nbytes: int):
+        if nbytes:
+            self._check(self.lib.zrt_d2d(dst_ptr, src_ptr, nbytes, self.stream), "d2d")
+
+    def download(self, t: Tensor) -> np.ndarray:
+        """Copy a device tensor to a new host array (synchronous)."""
+        out = np.empty(t.shape, dtype=NUMPY_OF[t.dtype])
+        if out.nbytes:
+            self._check(self.lib.zrt_d2h(out.ctypes.data, t.ptr, out.nbytes, self.stream, 0), "d2h")
+        return out
+
+    def download_f32(self, t: Tensor) -> np.ndarray:
+        a = self.download(t)
+        if t.dtype == BF16:
+            return (a.astype(np.uint32) << 16).view(np.float32)
+        return a.astype(np.float32, copy=False)
+
+    def sync(self):
+        self._check(self.lib.zrt_stream_sync(self.stream), "stream sync")
+
+    # -- events
+    def event(self) -> int:
+        e = C.c_void_p()
+        self._check(self.lib.zrt_event_create(C.byref(e)), "event create")
+        return e.value
+
+    def record(self, ev: int):
+        self._check(self.lib.zrt_event_record(ev, self.stream), "event record")
+
+    def wait_event(self, ev: int):
+        self._check(self.lib.zrt_event_sync(ev), "event sync")
+
+    def elapsed_ms(self, a: int, b: int) -> float:
+        self._check(self.lib.zrt_event_sync(b), "event sync")
+        ms = C.c_float()
+        self._check(self.lib.zrt_event_elapsed_ms(a, b, C.byref(ms)), "event elapsed")
+        return ms.value
+
+    # -- graphs
+    def capture_begin(self):
+        self._check(self.lib.zrt_capture_begin(self.stream), "capture begin")
+
+    def capture_end(self) -> int:
+        g = C.c_void_p()
+        self._check(self.lib.zrt_capture_end(self.stream, C.byref(g)), "capture end")
+        return g.value
+
+    def graph_launch(self, g: int):
+        self._check(self.lib.zrt_graph_launch(g, self.stream), "graph launch")
+
+    def graph_destroy(self, g: int):
+        self.lib.zrt_graph_destroy(g)

@@ -1,0 +1,60 @@
+"""Random-weights mode: a model folder (config.json, model.safetensors) from a
+configuration and a seed.
+
+Values are drawn on the host with a seeded generator, one stream per tensor
+name, so a tensor's values do not depend on the other tensors: matrices
+N(0, std), gains N(0, gain_std).  The reference has no such mode for models
+(random weights appear only in its adapter tests, orchestrator/lora_manager.py:157).
+"""
+from __future__ import annotations
+
+import json
+import os
+import zlib
+from typing import Optional
+
+import numpy as np
+
+from ..config.base import ARCHITECTURES, resolve_architecture
+from ..parts.base import ROLE_GAIN
+from . import safetensors as st
+from .loader import merge_reqs
+
+
+def random_tensors(reqs, seed: int, std: float, gain_std: float):
+    out = {}
+    for key, r in merge_reqs(reqs).items():
+        rng = np.random.Generator(np.random.Philox(key=[int(seed), zlib.crc32(key.encode())]))
+        s = r.init_std if r.init_std is not None else (gain_std if r.role == ROLE_GAIN else std)
+        out[r.name] = (rng.standard_normal(r.shape, dtype=np.float32) * np.float32(s))
+    return out
+
+
+def write_random_model(out_dir: str, config: dict, seed: int = 0, std: float = 0.02,
+                       gain_std: float = 0.1, dtype: str = "bfloat16") -> str:
+    """Write ``out_dir/config.json`` and ``out_dir/model.safetensors``.
+
+    ``config`` is a config.json dictionary (it must name its architecture);
+    ``dtype`` is the storage type of the file, "bfloat16" or "float32".
+    """
+    from .. import models  # noqa: F401  (registers architectures)
+    from ..engine.model import Model
+    arch = resolve_architecture(config)
+    typed = arch.config_from_dict(config)
+    model = Model(arch.plan(typed))
+    tensors = random_tensors(model.tensor_reqs(), seed, std, gain_std)
+    if dtype in ("bfloat16", "bf16"):
+        packed = {n: ("BF16", st.f32_to_bf16_bits(a)) for n, a in tensors.items()}
+    elif dtype in ("float32", "fp32"):
+        packed = {n: ("F32", a) for n, a in tensors.items()}
+    else:
+        raise ValueError(f"dtype must be bfloat16 or float32, got {dtype!r}")
+    os.makedirs(out_dir, exist_ok=True)
+    cfg = dict(config)
+    cfg.setdefault("architectures", [arch.name])
+    cfg["torch_dtype"] = "bfloat16" if dtype.startswith("b") else "float32"
+    with open(os.path.join(out_dir, "config.json"), "w") as f:
+        json.dump(cfg, f, indent=1)
+    st.write_file(os.path.join(out_dir, "model.safetensors"), packed,
+                  metadata={"format": "pt", "seed": seed})
+    return out_dir
