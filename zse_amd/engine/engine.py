@@ -1,0 +1,179 @@
+"""The Python entry point: a model folder in, generated token ids out.
+
+``Engine`` stands where the reference has ``ZSEEngine`` (one request at a time,
+orchestrator/engine.py:70-525) and ``ZStreamerEngine`` (continuous batching,
+zstreamer/engine.py:345-584): it owns the loaded model, the step runner with its
+cache, the scheduler and the sampler.  ``generate`` runs any number of prompts
+to completion; ``generate_tokens`` keeps the reference's single-prompt call and
+its return value of prompt plus generated tokens (orchestrator/engine.py:299-318).
+Prompts are token ids: text and tokenizers are outside this engine.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, Iterator, List, Optional, Sequence, Union
+
+from ..runtime.device import Runtime, canonical_dtype
+from ..sampling.sampler import DeviceSampler, SamplingParams, fresh_seed, uniform
+from .loading import load_model, random_model
+from .model import Model
+from .request import FinishReason, Request, RequestState
+from .runner import StepEntry, StepRunner
+from .scheduler import Scheduler, SchedulerConfig, StepPlan
+
+
+@dataclass
+class EngineStats:
+    steps: int = 0
+    prompt_tokens: int = 0
+    generated_tokens: int = 0
+    preemptions: int = 0
+    seconds: float = 0.0
+
+    @property
+    def tokens_per_second(self) -> float:
+        return self.generated_tokens / self.seconds if self.seconds > 0 else 0.0
+
+
+class Engine:
+    def __init__(self, model: Union[str, Model], dtype: str = "bfloat16", block_size: int = 16,
+                 num_blocks: Optional[int] = None, max_batch_tokens: int = 4096,
+                 max_batch_seqs: int = 64, prefill_chunk_size: int = 512,
+                 max_seq_len: Optional[int] = None, device_index: int = 0, tuned: bool = True,
+                 use_graphs: bool = True, quiet: bool = True):
+        self.rt = Runtime.get(device_index)
+        self.dtype = canonical_dtype(dtype)
+        self.model = load_model(model, self.dtype, self.rt) if isinstance(model, str) else model
+        max_len = min(max_seq_len or self.model.plan.max_position, self.model.plan.max_position)
+        if num_blocks is None:
+            # enough for every request slot at a moderate length, bounded by memory left
+            per_token = sum(2 * n.num_kv_heads * n.head_dim for n in self.model.cache_needs()
+                            if n is not None and hasattr(n, "num_kv_heads"))
+            per_token *= 2 if self.dtype == "bfloat16" else 4
+            free = self.rt.info().free_memory
+            want_tokens = max_batch_seqs * max_len
+            fit_tokens = int(free * 0.6) // max(per_token, 1)
+            num_blocks = max(1, min(want_tokens, fit_tokens) // block_size)
+        self.runner = StepRunner(self.model, self.rt, self.dtype, page_size=block_size,
+                                 num_pages=num_blocks, max_seqs=max_batch_seqs,
+                                 max_batch_tokens=max_batch_tokens, max_model_len=max_len,
+                                 tuned=tuned, use_graphs=use_graphs)
+        self.scheduler = Scheduler(SchedulerConfig(max_batch_tokens, prefill_chunk_size, max_batch_seqs),
+                                   self.runner.manager)
+        self.sampler = DeviceSampler(self.rt, self.runner.k, max_batch_seqs)
+        self._stats = EngineStats()
+        self._next_id = 0
+        self.quiet = quiet
+
+    # ---- requests
+    def add_request(self, prompt_tokens: Sequence[int], params: Optional[SamplingParams] = None,
+                    request_id=None) -> Request:
+        params = params or SamplingParams()
+        vocab = self.model.plan.vocab_size
+        for t in prompt_tokens:
+            if not (0 <= int(t) < vocab):
+                raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+        if request_id is None:
+            request_id = f"req-{self._next_id}"
+        self._next_id += 1
+        req = Request(request_id, [int(t) for t in prompt_tokens], params,
+                      seed=params.seed if params.seed is not None else fresh_seed())
+        self.scheduler.add_request(req)
+        self._stats.prompt_tokens += len(req.prompt_tokens)
+        return req
+
+    def step(self) -> List[Request]:
+        """Schedule, run and sample one step; returns the requests that finished in it."""
+        plan = self.scheduler.schedule()
+        if not plan:
+            return list(plan.failed)
+        entries = [StepEntry(s.request.request_id,
+                             s.request.all_tokens[s.start:s.start + s.count],
+                             [s.count - 1] if s.sample else []) for s in plan.items]
+        logits = self.runner.step(entries, download=False)
+        rows = []
+        who = []
+        for s in plan.items:
+            if s.sample:
+                r = s.request
+                rows.append({"params": r.params, "u": uniform(r.seed, len(r.output_tokens)),
+                             "past": set(r.all_tokens) if r.params.repetition_penalty != 1.0 else ()})
+                who.append(r.request_id)
+        ids = self.sampler.sample(logits, rows) if rows else []
+        done = self.scheduler.on_step_done(plan, dict(zip(who, ids)))
+        self._stats.steps += 1
+        self._stats.generated_tokens += len(ids)
+        self._stats.preemptions = self.scheduler.num_preemptions
+        return done + list(plan.failed)
+
+    def run(self) -> None:
+        t0 = time.monotonic()
+        while self.scheduler.has_work():
+            self.step()
+        self._stats.seconds += time.monotonic() - t0
+
+    # ---- the calls users make
+    def generate(self, prompts: Sequence[Sequence[int]],
+                 params: Union[None, SamplingParams, Sequence[SamplingParams]] = None) -> List[List[int]]:
+        """Generated token ids for each prompt (the prompt itself is not repeated).
+        A request that could not be served raises ``RuntimeError``."""
+        if params is None or isinstance(params, SamplingParams):
+            plist = [params or SamplingParams()] * len(prompts)
+        else:
+            plist = list(params)
+            if len(plist) != len(prompts):
+                raise ValueError("one SamplingParams per prompt, or one for all")
+        reqs = []
+        for p, sp in zip(prompts, plist):
+            if sp.max_tokens == 0:
+                reqs.append(None)
+                continue
+            reqs.append(self.add_request(p, sp))
+        self.run()
+        out = []
+        for r in reqs:
+            if r is None:
+                out.append([])
+                continue
+            if r.finish_reason == FinishReason.ERROR:
+                raise RuntimeError(f"request {r.request_id}: {r.error}")
+            out.append(list(r.output_tokens))
+        return out
+
+    def generate_tokens(self, token_ids: Sequence[int], max_tokens: int = 128, temperature: float = 1.0,
+                        top_p: float = 1.0, top_k: int = 0, repetition_penalty: float = 1.0,
+                        stop_tokens: Optional[List[int]] = None, seed: Optional[int] = None) -> List[int]:
+        """Prompt plus generated tokens of one request (orchestrator/engine.py:299-318)."""
+        sp = SamplingParams(max_tokens, temperature, top_p, top_k, repetition_penalty, stop_tokens, seed)
+        return list(token_ids) + self.generate([token_ids], sp)[0]
+
+    def stream_generate_tokens(self, token_ids: Sequence[int], **kw) -> Iterator[int]:
+        """Generated tokens of one request as they are produced (orchestrator/engine.py:320-367)."""
+        sp = SamplingParams(**kw)
+        if sp.max_tokens == 0:
+            return
+        req = self.add_request(token_ids, sp)
+        seen = 0
+        while not req.finished:
+            self.step()
+            while seen < len(req.output_tokens):
+                yield req.output_tokens[seen]
+                seen += 1
+        if req.finish_reason == FinishReason.ERROR:
+            raise RuntimeError(f"request {req.request_id}: {req.error}")
+
+    def stats(self) -> EngineStats:
+        return self._stats
+
+    def close(self) -> None:
+        self.runner = None
+        self.sampler = None
+
+    destroy = close
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()

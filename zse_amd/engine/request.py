@@ -1,0 +1,62 @@
+"""A request's record through its life.
+
+States and finish reasons follow the reference (zstreamer/request.py:18-35):
+WAITING -> PREFILLING -> DECODING -> FINISHED, with PREEMPTED for a request
+whose pages were taken and which waits to be computed again.  ``num_computed``
+stands where the reference has ``prefill_offset`` and also covers that
+recomputation: it counts the tokens of ``prompt + output`` whose keys are in
+the cache.
+"""
+from __future__ import annotations
+
+import enum
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+from ..sampling.sampler import SamplingParams
+
+
+class RequestState(enum.Enum):
+    WAITING = "waiting"
+    PREFILLING = "prefilling"
+    DECODING = "decoding"
+    PREEMPTED = "preempted"
+    FINISHED = "finished"
+
+
+class FinishReason(enum.Enum):
+    LENGTH = "length"     # max_tokens, or the model's longest context, reached
+    STOP = "stop"         # a stop token was produced
+    ERROR = "error"       # the request cannot be served (it does not fit the cache alone)
+
+
+@dataclass
+class Request:
+    request_id: object
+    prompt_tokens: List[int]
+    params: SamplingParams = field(default_factory=SamplingParams)
+    seed: int = 0
+    state: RequestState = RequestState.WAITING
+    output_tokens: List[int] = field(default_factory=list)
+    num_computed: int = 0
+    finish_reason: Optional[FinishReason] = None
+    error: Optional[str] = None
+    arrival: int = 0
+    num_preemptions: int = 0
+
+    @property
+    def all_tokens(self) -> List[int]:
+        return self.prompt_tokens + self.output_tokens
+
+    @property
+    def num_tokens(self) -> int:
+        return len(self.prompt_tokens) + len(self.output_tokens)
+
+    @property
+    def remaining(self) -> int:
+        """Tokens known but not yet in the cache."""
+        return self.num_tokens - self.num_computed
+
+    @property
+    def finished(self) -> bool:
+        return self.state == RequestState.FINISHED

@@ -1,0 +1,1 @@
+from .sampler import DeviceSampler, SamplingParams, fresh_seed, sample_host, uniform

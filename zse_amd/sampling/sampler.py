@@ -1,0 +1,158 @@
+"""Choosing the next token: greedy, temperature, top-k, top-p, repetition penalty.
+
+Option names, meanings and the order of operations are the reference's
+(orchestrator/sampler.py:33-98; orchestrator/engine.py:37-46): repetition penalty,
+then the greedy test (temperature <= 0 or < 1e-6), temperature, top-k (ties at
+the threshold stay, :146-156), top-p (smallest set by descending probability
+whose mass reaches p, :186-203), softmax with the maximum subtracted
+(:168-173), and the first index whose running sum exceeds a uniform number
+(:205-213).  Two things differ on purpose: top_k and top_p are off unless
+given, and the uniform number is a pure function of (seed, index of the
+output token) instead of coming from one shared generator (:30-31), so a
+request samples the same tokens whatever else is in the batch.
+
+Greedy and plain temperature sampling run on the device
+(csrc/sampling.hip); rows that use top-k, top-p or a penalty are brought to the
+host, where the reference samples everything (:10-11).
+"""
+from __future__ import annotations
+
+import math
+import os
+from dataclasses import dataclass, field
+from typing import Dict, Iterable, List, Optional, Sequence
+
+import numpy as np
+
+_MASK = (1 << 64) - 1
+
+
+@dataclass
+class SamplingParams:
+    max_tokens: int = 128
+    temperature: float = 1.0          # <= 0 (or < 1e-6): greedy
+    top_p: float = 1.0                # 1.0: off
+    top_k: int = 0                    # 0: off
+    repetition_penalty: float = 1.0   # 1.0: off
+    stop_tokens: Optional[List[int]] = None
+    seed: Optional[int] = None
+
+    def __post_init__(self):
+        if self.max_tokens < 0:
+            raise ValueError("max_tokens must not be negative")
+        if not (0.0 < self.top_p <= 1.0):
+            raise ValueError("top_p must be in (0, 1]")
+        if self.top_k < 0:
+            raise ValueError("top_k must not be negative")
+        if self.repetition_penalty <= 0:
+            raise ValueError("repetition_penalty must be positive")
+
+    @property
+    def greedy(self) -> bool:
+        return self.temperature <= 0 or self.temperature < 1e-6
+
+    @property
+    def on_device(self) -> bool:
+        """True when the device kernels cover this request's sampling."""
+        return self.repetition_penalty == 1.0 and (self.greedy or (self.top_k == 0 and self.top_p >= 1.0))
+
+
+def _mix64(z: int) -> int:
+    z = (z + 0x9E3779B97F4A7C15) & _MASK
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK
+    return z ^ (z >> 31)
+
+
+def uniform(seed: int, index: int) -> float:
+    """A number in [0, 1) that depends only on the request's seed and on which of
+    its output tokens is being drawn."""
+    return (_mix64(_mix64(int(seed) & _MASK) ^ ((int(index) * 0xD1342543DE82EF95) & _MASK)) >> 11) / float(1 << 53)
+
+
+def fresh_seed() -> int:
+    return int.from_bytes(os.urandom(8), "little")
+
+
+# ---------------------------------------------------------------- host sampling
+
+def apply_repetition_penalty(z: np.ndarray, past: Iterable[int], penalty: float) -> np.ndarray:
+    counts: Dict[int, int] = past if isinstance(past, dict) else {int(t): 1 for t in past}
+    for tid, cnt in counts.items():
+        if 0 <= tid < len(z):
+            s = penalty ** (1.0 + math.log2(cnt)) if cnt > 1 else penalty
+            z[tid] = z[tid] / s if z[tid] > 0 else z[tid] * s
+    return z
+
+
+def sample_host(logits: np.ndarray, params: SamplingParams, u: float, past: Iterable[int] = ()) -> int:
+    z = np.array(logits, dtype=np.float64)
+    if params.repetition_penalty != 1.0 and past:
+        z = apply_repetition_penalty(z, past, params.repetition_penalty)
+    if params.greedy:
+        return int(np.argmax(z))
+    z *= 1.0 / params.temperature
+    if 0 < params.top_k < len(z):
+        thr = np.partition(z, len(z) - params.top_k)[len(z) - params.top_k]
+        z[z < thr] = -np.inf
+    if params.top_p < 1.0:
+        e = np.exp(z - z.max())
+        pr = e / e.sum()
+        order = np.argsort(-pr, kind="stable")
+        cum = np.cumsum(pr[order])
+        keep_n = int(np.searchsorted(cum, params.top_p, side="left")) + 1
+        mask = np.ones(len(z), dtype=bool)
+        mask[order[:keep_n]] = False
+        z[mask] = -np.inf
+    e = np.exp(z - z.max())
+    cum = np.cumsum(e / e.sum())
+    return min(int(np.searchsorted(cum, u, side="right")), len(z) - 1)
+
+
+# ---------------------------------------------------------------- device sampling
+
+class DeviceSampler:
+    """Runs the argmax and inverse-CDF kernels on logits that are still on the device."""
+
+    def __init__(self, rt, kernels, max_rows: int):
+        from ..runtime.device import F32, F64, I32
+        self.rt = rt
+        self.k = kernels
+        self.max_rows = max_rows
+        self.ids = rt.empty((max_rows,), I32)
+        self.ids2 = rt.empty((max_rows,), I32)
+        self.temp = rt.empty((max_rows,), F32)
+        self.u = rt.empty((max_rows,), F64)
+
+    def sample(self, logits, rows: Sequence[dict]) -> List[int]:
+        """``logits``: device float32 [n, vocab]; ``rows``: per row a dict with
+        ``params``, ``u`` and ``past``.  Returns the chosen ids."""
+        n, V = logits.shape
+        if n == 0:
+            return []
+        if n > self.max_rows:
+            raise ValueError(f"{n} rows to sample, room for {self.max_rows}")
+        rt, k = self.rt, self.k
+        need_greedy = any(r["params"].on_device and r["params"].greedy for r in rows)
+        need_temp = any(r["params"].on_device and not r["params"].greedy for r in rows)
+        need_host = [i for i, r in enumerate(rows) if not r["params"].on_device]
+        out: List[Optional[int]] = [None] * n
+        if need_greedy:
+            k.zk_argmax(logits.ptr, self.ids.ptr, n, V, rt.stream)
+        if need_temp:
+            t = np.array([r["params"].temperature if not r["params"].greedy else 1.0 for r in rows],
+                         dtype=np.float32)
+            u = np.array([r["u"] for r in rows], dtype=np.float64)
+            rt.copy_h2d(self.temp.ptr, t)
+            rt.copy_h2d(self.u.ptr, u)
+            k.zk_sample(logits.ptr, self.temp.ptr, self.u.ptr, None, self.ids2.ptr, n, V, rt.stream)
+        g = rt.download(self.ids.rows(0, n)) if need_greedy else None
+        s = rt.download(self.ids2.rows(0, n)) if need_temp else None
+        for i, r in enumerate(rows):
+            p = r["params"]
+            if p.on_device:
+                out[i] = int(g[i]) if p.greedy else int(s[i])
+        for i in need_host:
+            row = rt.download(logits.rows(i, i + 1))[0]
+            out[i] = sample_host(row, rows[i]["params"], rows[i]["u"], rows[i].get("past", ()))
+        return out

@@ -112,7 +112,7 @@ def to_float32(arr: np.ndarray, dtype_tag: str) -> np.ndarray:
     """Any stored float tensor as float32 values."""
     if dtype_tag == "BF16":
         return bf16_bits_to_f32(arr)
-    return np.asarray(arr, dtype=np.float32)
+    return np.array(arr, dtype=np.float32)      # a copy: the caller may rewrite the file
 
 
 def read_folder_f32(model_dir: str) -> Dict[str, np.ndarray]:
