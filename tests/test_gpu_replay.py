@@ -1,0 +1,153 @@
+"""The engine against the plain implementation under every way of cutting the work:
+whole, most of it then the last 32 one by one, portions of changing size, and mixed
+batches with so few pages that they are used again; in float32 and in bfloat16."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from conftest import ROOT, TINY, random_tokens
+from gpu_util import (assert_close, chunked_steps, make_runner, mixed_steps, reference_for, run_steps,
+                      tail_decode_steps, whole_steps)
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [50, 77, 37, 23, 64, 41], "B": [90, 40, 57, 33, 120, 66]}
+PAGE = {"A": 4, "B": 8}
+
+
+def streams_of(name):
+    V = TINY[name][0]["vocab_size"]
+    return {f"r{i}": random_tokens(V, n, 100 + i) for i, n in enumerate(LENGTHS[name])}
+
+
+@pytest.fixture(scope="module")
+def cases(tiny_folders):
+    out = {}
+    for name in ("A", "B"):
+        for dtype in ("float32", "bfloat16"):
+            folder = tiny_folders[(name, dtype)]
+            streams = streams_of(name)
+            refs = {r: reference_for(name, dtype, folder, t) for r, t in streams.items()}
+            out[(name, dtype)] = (folder, streams, refs)
+    return out
+
+
+def check(rows, refs, dtype, what):
+    assert set(rows) == set(refs)
+    for r in refs:
+        assert_close(rows[r], refs[r], dtype, f"{what} {r}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_every_split_matches_the_plain_implementation(cases, name, dtype):
+    folder, streams, refs = cases[(name, dtype)]
+    longest = max(len(t) for t in streams.values())
+    runner = make_runner(folder, dtype, page_size=PAGE[name], cache_tokens=-(-longest // 64) * 64,
+                         max_seqs=4, max_batch_tokens=256, max_model_len=256)
+    whole = run_steps(runner, streams, whole_steps(streams))
+    check(whole, refs, dtype, "whole")
+    tail = run_steps(runner, streams, tail_decode_steps(streams))
+    check(tail, refs, dtype, "last 32 one by one")
+    chunk = run_steps(runner, streams, chunked_steps(streams))
+    check(chunk, refs, dtype, "portions")
+    for r in streams:
+        if dtype == "float32":
+            # every sum runs in an order fixed by positions alone: the cuts change nothing
+            assert np.array_equal(whole[r], tail[r]) and np.array_equal(whole[r], chunk[r]), r
+    assert all(p.free_pages == p.num_pages for p in runner.manager.pools)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_mixed_batches_with_pages_used_again(cases, name, dtype):
+    folder, streams, refs = cases[(name, dtype)]
+    # room for the four longest live requests, each rounded up to 64: far less than all six
+    top4 = sorted((len(t) for t in streams.values()), reverse=True)[:4]
+    pool = sum(-(-n // 64) * 64 for n in top4)
+    assert pool < sum(-(-len(t) // PAGE[name]) * PAGE[name] for t in streams.values()) + 64
+    runner = make_runner(folder, dtype, page_size=PAGE[name], cache_tokens=pool, max_seqs=4,
+                         max_batch_tokens=256, max_model_len=256)
+    seen_pages = set()
+    for seed in (0, 1):
+        steps = mixed_steps(streams, seed=seed)
+        assert max(len(e) for e, _ in steps) == 4
+        assert any(any(n > 1 for _, n in e) and any(n == 1 for _, n in e) for e, _ in steps)
+        rows = run_steps(runner, streams, steps)
+        check(rows, refs, dtype, f"mixed seed {seed}")
+        assert all(p.free_pages == p.num_pages for p in runner.manager.pools)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_window_release_lets_a_small_pool_serve_a_long_request(cases, dtype):
+    # the all-keys group needs every page; give the pool exactly that and decode far past
+    # the window: sliding layers hand pages back while the request is still running
+    name = "A"
+    folder, _, _ = cases[(name, dtype)]
+    toks = random_tokens(TINY[name][0]["vocab_size"], 200, 9)
+    ref = reference_for(name, dtype, folder, toks)
+    runner = make_runner(folder, dtype, page_size=4, cache_tokens=200, max_seqs=2, max_batch_tokens=64,
+                         max_model_len=256)
+    steps = [([("x", 40)], [])] + [([("x", 1)], []) for _ in range(160)]
+    rows = run_steps(runner, {"x": toks}, steps)
+    assert_close(rows["x"], ref, dtype, "long decode")
+    m = runner.manager
+    sliding, full = m.pools[0], m.pools[1]
+    assert full.used_pages == 50 and sliding.used_pages <= 3      # window 8, pages of 4
+    runner.finish("x")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(cases, dtype):
+    name = "B"
+    folder, streams, refs = cases[(name, dtype)]
+    runner = make_runner(folder, dtype, page_size=8, cache_tokens=64, max_seqs=4, max_batch_tokens=64,
+                         max_model_len=64)
+    t = streams["r0"][:3]
+    ref = refs["r0"][:3]
+    rows = run_steps(runner, {"a": t}, [([("a", 1)], []), ([("a", 1)], []), ([("a", 1)], ["a"])])
+    assert_close(rows["a"], ref, dtype, "one by one from the first token")
+    rows = run_steps(runner, {"a": t[:1]}, [([("a", 1)], ["a"])])
+    assert_close(rows["a"], ref[:1], dtype, "a prompt of one token")
+
+
+def test_trace_run_program(cases, tmp_path):
+    """bin/trace_run as a user starts it: JSON steps on stdin, <step>.f32 files out."""
+    name, dtype = "A", "float32"
+    folder, streams, refs = cases[(name, dtype)]
+    steps = mixed_steps(streams, seed=3)
+    fed = {r: 0 for r in streams}
+    lines, wants = [], []
+    for i, (entries, ends) in enumerate(steps):
+        es = []
+        for r, n in entries:
+            want = [n - 1] if i % 3 else list(range(n))
+            if i % 7 == 5:
+                want = []
+            es.append({"id": r, "tokens": streams[r][fed[r]:fed[r] + n], "want": want})
+            wants.append((i, r, [fed[r] + w for w in want]))
+            fed[r] += n
+        lines.append(json.dumps({"step": i, "entries": es, "end": ends}))
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder,
+                        "--dtype", dtype, "--out", str(out), "--max-tokens", "256", "--block-size", "4"],
+                       input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert p.stdout.split("\n")[:len(steps)] == [f"done {i}" for i in range(len(steps))]
+    V = TINY[name][0]["vocab_size"]
+    by_step = {}
+    for i, r, pos in wants:
+        by_step.setdefault(i, []).extend((r, q) for q in pos)
+    for i, items in by_step.items():
+        path = out / f"{i}.f32"
+        if not items:
+            assert not path.exists()
+            continue
+        z = np.fromfile(path, dtype="<f4").reshape(-1, V)
+        assert z.shape[0] == len(items)
+        for row, (r, q) in zip(z, items):
+            assert_close(row, refs[r][q], dtype, f"trace_run step {i} {r}@{q}")
