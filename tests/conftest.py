@@ -40,7 +40,9 @@ def tiny_folders(tmp_path_factory):
     for name, (cfg, seed, std, gstd) in TINY.items():
         for dtype in ("float32", "bfloat16"):
             d = str(tmp_path_factory.mktemp(f"tiny{name}_{dtype}"))
-            write_random_model(d, cfg, seed=seed, std=std, gain_std=gstd, dtype=dtype)
+            # a small embedding keeps the tied head from simply echoing the last token
+            write_random_model(d, cfg, seed=seed, std=std, gain_std=gstd, dtype=dtype,
+                               std_of={"embed_tokens": std / 4})
             out[(name, dtype)] = d
     return out
 

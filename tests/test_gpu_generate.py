@@ -1,0 +1,140 @@
+"""Generation through the entry points: ``Engine.generate`` and the ``zse generate`` command
+against a greedy loop over the plain implementation; sampled requests against the plain
+sampler on the engine's own logits."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from conftest import ROOT, TINY, random_tokens, read_weights
+from plain import gemma2_plain as P
+
+pytestmark = pytest.mark.gpu
+
+
+def plain_greedy(cfg, w, prompt, n, margin_log=None):
+    toks = list(prompt)
+    for _ in range(n):
+        z = P.forward(cfg, w, toks, np.float64)[-1]
+        if margin_log is not None:
+            s = np.sort(z)
+            margin_log.append(s[-1] - s[-2])
+        toks.append(int(np.argmax(z)))
+    return toks[len(prompt):]
+
+
+@pytest.mark.parametrize("name,lengths,n_new", [("A", (5, 11, 17), 8), ("B", (1, 9, 23, 40), 12)])
+def test_greedy_generation_float32(tiny_folders, name, lengths, n_new):
+    from zse_amd.engine.engine import Engine
+    from zse_amd.sampling import SamplingParams
+    cfg = TINY[name][0]
+    folder = tiny_folders[(name, "float32")]
+    w = read_weights(folder)
+    prompts = [random_tokens(cfg["vocab_size"], n, 40 + n) for n in lengths]
+    eng = Engine(folder, dtype="float32", block_size=4 if name == "A" else 8, num_blocks=64,
+                 max_batch_tokens=32, max_batch_seqs=4, prefill_chunk_size=4 if name == "A" else 7,
+                 max_seq_len=128)
+    got = eng.generate(prompts, SamplingParams(max_tokens=n_new, temperature=0.0))
+    for p, g in zip(prompts, got):
+        assert g == plain_greedy(cfg, w, p, n_new)
+    assert eng.stats().generated_tokens == n_new * len(prompts)
+    # one prompt, the reference's call shape: prompt plus generated tokens come back
+    both = eng.generate_tokens(prompts[0], max_tokens=3, temperature=0.0)
+    assert both == prompts[0] + got[0][:3]
+    assert list(eng.stream_generate_tokens(prompts[1], max_tokens=4, temperature=0.0)) == got[1][:4]
+    eng.close()
+
+
+def test_greedy_generation_bfloat16(tiny_folders):
+    from zse_amd.engine.engine import Engine
+    from zse_amd.sampling import SamplingParams
+    cfg = TINY["A"][0]
+    folder = tiny_folders[("A", "bfloat16")]
+    w = read_weights(folder)
+    prompts = [random_tokens(512, n, 60 + n) for n in (5, 11, 17)]
+    eng = Engine(folder, dtype="bfloat16", block_size=4, num_blocks=64, max_batch_tokens=32,
+                 max_batch_seqs=4, prefill_chunk_size=4, max_seq_len=128)
+    got = eng.generate(prompts, SamplingParams(max_tokens=8, temperature=0.0))
+    eng.close()
+    for p, g in zip(prompts, got):
+        toks = list(p)
+        for i, t in enumerate(g):
+            z = P.forward(cfg, w, toks, np.float64)[-1]
+            s = np.sort(z)
+            assert t == int(np.argmax(z)) or s[-1] - s[-2] < 0.05, f"token {i} of {p}"
+            toks.append(t)
+
+
+def test_sampled_requests_do_not_depend_on_the_batch(tiny_folders):
+    """Temperature 0.8 with seed 7: the same tokens alone, in a batch, under another chunk size
+    and after a forced recomputation; each token is what the plain sampler draws from the
+    engine's own logits."""
+    from zse_amd.engine.engine import Engine
+    from zse_amd.engine.runner import StepEntry
+    from zse_amd.sampling import SamplingParams, uniform
+    cfg = TINY["B"][0]
+    folder = tiny_folders[("B", "float32")]
+    prompts = [random_tokens(1000, n, 80 + n) for n in (1, 9, 23, 40)]
+    params = [SamplingParams(max_tokens=12, temperature=0.0), SamplingParams(max_tokens=12, temperature=0.8, seed=7),
+              SamplingParams(max_tokens=12, temperature=0.0), SamplingParams(max_tokens=12, temperature=0.8, seed=7)]
+
+    def run(chunk, seqs, blocks, which):
+        eng = Engine(folder, dtype="float32", block_size=8, num_blocks=blocks, max_batch_tokens=64,
+                     max_batch_seqs=seqs, prefill_chunk_size=chunk, max_seq_len=128)
+        out = eng.generate([prompts[i] for i in which], [params[i] for i in which])
+        st = eng.stats()
+        eng.close()
+        return out, st
+
+    batch, _ = run(7, 4, 64, [0, 1, 2, 3])
+    alone = [run(16, 1, 64, [i])[0][0] for i in range(4)]
+    assert batch == alone
+    tight, st = run(5, 4, 13, [0, 1, 2, 3])        # 13 pages of 8: pages run out while decoding
+    assert st.preemptions > 0 and tight == batch
+    # each sampled token is the plain sampler's draw on logits of the same position
+    from gpu_util import make_runner
+    runner = make_runner(folder, "float32", page_size=8, cache_tokens=128, max_seqs=2,
+                         max_batch_tokens=128, max_model_len=128)
+    seq = prompts[3] + batch[3]
+    z = runner.step([StepEntry("s", seq, list(range(len(seq))))])
+    for i, tok in enumerate(batch[3]):
+        assert tok == P.sample(z[len(prompts[3]) - 1 + i], uniform(7, i), temperature=0.8)
+
+
+def test_top_k_top_p_and_penalty_rows_go_through_the_host_sampler(tiny_folders):
+    from zse_amd.engine.engine import Engine
+    from zse_amd.sampling import SamplingParams
+    folder = tiny_folders[("A", "float32")]
+    prompt = random_tokens(512, 9, 5)
+    eng = Engine(folder, dtype="float32", block_size=4, num_blocks=64, max_batch_tokens=32,
+                 max_batch_seqs=4, prefill_chunk_size=8, max_seq_len=64)
+    greedy = eng.generate([prompt], SamplingParams(max_tokens=6, temperature=0.0))[0]
+    k1 = eng.generate([prompt], SamplingParams(max_tokens=6, temperature=1.0, top_k=1, seed=3))[0]
+    assert k1 == greedy                                     # top-1 sampling is greedy
+    p_small = eng.generate([prompt], SamplingParams(max_tokens=6, temperature=1.0, top_p=1e-6, seed=3))[0]
+    assert p_small == greedy
+    pen = eng.generate([prompt], SamplingParams(max_tokens=6, temperature=0.0, repetition_penalty=50.0))[0]
+    assert len(set(pen) | set(prompt)) == len(pen) + len(set(prompt))     # nothing is repeated
+    stop = eng.generate([prompt], SamplingParams(max_tokens=6, temperature=0.0, stop_tokens=[greedy[-1]]))[0]
+    assert stop == greedy[:greedy.index(greedy[-1]) + 1]
+    eng.close()
+
+
+def test_zse_generate_command(tiny_folders, tmp_path):
+    from zse_amd.engine.engine import Engine
+    cfg = TINY["A"][0]
+    folder = tiny_folders[("A", "float32")]
+    w = read_weights(folder)
+    prompts = [random_tokens(512, n, 90 + n) for n in (6, 13)]
+    f = tmp_path / "prompts.txt"
+    f.write_text("\n".join(" ".join(map(str, p)) for p in prompts) + "\n")
+    p = subprocess.run([sys.executable, "-m", "zse_amd", "generate", folder, "--prompt-ids-file", str(f),
+                        "--max-tokens", "5", "--temperature", "0", "--dtype", "float32",
+                        "--block-size", "4", "--num-blocks", "64", "--prefill-chunk-size", "4",
+                        "--max-seq-len", "64", "--quiet"],
+                       capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = [list(map(int, l.split())) for l in p.stdout.strip().split("\n")]
+    assert lines == [plain_greedy(cfg, w, q, 5) for q in prompts]

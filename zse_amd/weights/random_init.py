@@ -21,28 +21,32 @@ from . import safetensors as st
 from .loader import merge_reqs
 
 
-def random_tensors(reqs, seed: int, std: float, gain_std: float):
+def random_tensors(reqs, seed: int, std: float, gain_std: float, std_of=None):
     out = {}
     for key, r in merge_reqs(reqs).items():
         rng = np.random.Generator(np.random.Philox(key=[int(seed), zlib.crc32(key.encode())]))
         s = r.init_std if r.init_std is not None else (gain_std if r.role == ROLE_GAIN else std)
+        for part, v in (std_of or {}).items():
+            if part in r.name:
+                s = v
         out[r.name] = (rng.standard_normal(r.shape, dtype=np.float32) * np.float32(s))
     return out
 
 
 def write_random_model(out_dir: str, config: dict, seed: int = 0, std: float = 0.02,
-                       gain_std: float = 0.1, dtype: str = "bfloat16") -> str:
+                       gain_std: float = 0.1, dtype: str = "bfloat16", std_of=None) -> str:
     """Write ``out_dir/config.json`` and ``out_dir/model.safetensors``.
 
     ``config`` is a config.json dictionary (it must name its architecture);
-    ``dtype`` is the storage type of the file, "bfloat16" or "float32".
+    ``dtype`` is the storage type of the file, "bfloat16" or "float32";
+    ``std_of`` maps a part of a tensor name to the deviation of the tensors that carry it.
     """
     from .. import models  # noqa: F401  (registers architectures)
     from ..engine.model import Model
     arch = resolve_architecture(config)
     typed = arch.config_from_dict(config)
     model = Model(arch.plan(typed))
-    tensors = random_tensors(model.tensor_reqs(), seed, std, gain_std)
+    tensors = random_tensors(model.tensor_reqs(), seed, std, gain_std, std_of)
     if dtype in ("bfloat16", "bf16"):
         packed = {n: ("BF16", st.f32_to_bf16_bits(a)) for n, a in tensors.items()}
     elif dtype in ("float32", "fp32"):
