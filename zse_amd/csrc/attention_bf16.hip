@@ -1,0 +1,332 @@
+// Paged attention on the matrix cores, bfloat16 in, float softmax.
+//
+// One kernel serves prompt portions and decoded tokens.  A wave owns up to 32
+// query rows: TPW consecutive tokens of one request times the g = nh / nkv
+// query heads that share a KV head, so every K and V tile it loads serves the
+// whole group (the reference's paged_attention_v2 stages a K/V tile once for
+// the heads of a group too, orchestrator/kernels.py:687-854, but is never
+// launched; the launched kernels read K and V once per query head and hold one
+// score per cached token in shared memory, :524-671, :859-958).
+//
+// Per tile of 32 keys:
+//   S^T[key, row]  = K[key, :] . Q[row, :]        32x32x16 MFMA, hd/16 steps
+//   scale, soft cap, mask (key <= pos, pos - key < window), running max / sum
+//   O^T[d, row]   += V^T[d, key] * P^T[key, row]  32x32x16 MFMA, 2 per 32 channels
+// S^T and O^T both keep a query row in a fixed lane (column = lane % 32), so the
+// running maximum, sum and rescale are per-lane scalars, and the probabilities
+// a lane holds after the first product are exactly its operand for the second:
+// the contraction order over keys is permuted to match (slots e < 4 of lane half
+// h are keys 4h + e, slots e >= 4 are keys 8 + 4h + e - 4), and V is read with
+// the same permutation.  V is therefore cached transposed, [page][kv head][hd][bs],
+// so that four consecutive keys of a channel are one 8-byte load.
+//
+// Decoded tokens use the split variant: the keys are cut into chunks of 128
+// aligned to absolute positions, one wave per chunk writes (max, sum, O) and a
+// second kernel joins the chunks in order; the cut does not depend on the batch.
+#include "common.h"
+
+#if ZSE_ACT_BF16
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define ATT_CHUNK 128
+
+struct AttnParams {
+  const __bf16* q;
+  int q_stride;
+  const __bf16* kcache;   // [page][nkv][bs][hd]
+  const __bf16* vcache;   // [page][nkv][hd][bs]
+  const int* block_table;
+  int max_blocks;
+  const int* q_start;     // [R + 1]
+  const int* ctx_len;     // [R]
+  __bf16* out;            // [T][nh][hd]
+  float* part_o;          // split: [slot][hd]
+  float* part_ml;         // split: [slot][2]
+  int nh, nkv, hd, bs;
+  float scale, softcap;
+  int window;
+  int tpw;                // tokens a wave owns
+  int r_begin;            // first request of this launch
+  int nchunks;            // split: chunks the grid covers
+};
+
+__device__ __forceinline__ float fast_tanh(float x) {
+  // tanh(x) = 1 - 2 / (exp(2x) + 1); exact at the ends, relative error ~1e-6 between
+  const float e = __expf(2.f * x);
+  return 1.f - 2.f / (e + 1.f);
+}
+
+template <int HD16, bool SPLIT>
+__global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
+  constexpr int DT = (HD16 + 1) / 2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lr = lane & 31, lk = lane >> 5;
+  const int r = p.r_begin + blockIdx.z;
+  const int kvh = blockIdx.y;
+  const int qs = p.q_start[r], n = p.q_start[r + 1] - qs;
+  if (n <= 0) return;
+  const int start = p.ctx_len[r] - n;
+  const int gi = SPLIT ? 0 : blockIdx.x * 4 + wave;
+  const int chunk = SPLIT ? blockIdx.x * 4 + wave : 0;
+  const int t0 = gi * p.tpw;
+  if (t0 >= n) return;
+  const int g = p.nh / p.nkv;
+  const int tok = lr / g, hq = lr - tok * g;
+  const int ntok = min(p.tpw, n - t0);
+  const bool row_ok = tok < ntok;
+  const int trow = qs + t0 + (row_ok ? tok : 0);
+  const int pos = start + t0 + (row_ok ? tok : 0);
+  const int head = kvh * g + (row_ok ? hq : 0);
+  const int pos_lo = start + t0, pos_hi = start + t0 + ntok - 1;
+  int key_lo = p.window > 0 ? max(0, pos_lo - p.window + 1) : 0;
+  int key_hi = pos_hi;
+  if (SPLIT) {
+    key_lo = max(key_lo, chunk * ATT_CHUNK);
+    key_hi = min(key_hi, chunk * ATT_CHUNK + ATT_CHUNK - 1);
+  }
+  if (key_lo > key_hi) return;
+  const int row_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int* table = p.block_table + (size_t)r * p.max_blocks;
+  const int hd = p.hd, bs = p.bs, nkv = p.nkv;
+
+  bf16x8 qf[HD16];
+  {
+    const __bf16* qr = p.q + (size_t)trow * p.q_stride + (size_t)head * hd + lk * 8;
+#pragma unroll
+    for (int ks = 0; ks < HD16; ks++) {
+      if (row_ok) qf[ks] = *(const bf16x8*)(qr + ks * 16);
+      else
+#pragma unroll
+        for (int e = 0; e < 8; e++) qf[ks][e] = (__bf16)0.f;
+    }
+  }
+  f32x16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) o[dt][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  for (int key0 = (key_lo / 32) * 32; key0 <= key_hi; key0 += 32) {
+    // ---- S^T = K Q^T
+    f32x16 s;
+#pragma unroll
+    for (int e = 0; e < 16; e++) s[e] = 0.f;
+    {
+      const int kk = min(key0 + lr, key_hi);
+      const int page = max(table[kk / bs], 0);
+      const __bf16* kr = p.kcache + (((size_t)page * nkv + kvh) * bs + (kk % bs)) * hd + lk * 8;
+      bf16x8 kf[HD16];
+#pragma unroll
+      for (int ks = 0; ks < HD16; ks++) kf[ks] = *(const bf16x8*)(kr + ks * 16);
+#pragma unroll
+      for (int ks = 0; ks < HD16; ks++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], s, 0, 0, 0);
+    }
+    // ---- V^T pieces for this tile (issued early; used after the softmax)
+    bf16x8 vf[DT][2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const int ka = min(key0 + h * 16 + 4 * lk, key_hi & ~3), kb = min(key0 + h * 16 + 8 + 4 * lk, key_hi & ~3);
+      const int pa = max(table[ka / bs], 0), pb = max(table[kb / bs], 0);
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++) {
+        const int d = min(dt * 32 + lr, hd - 1);
+        const bf16x4 va = *(const bf16x4*)(p.vcache + (((size_t)pa * nkv + kvh) * hd + d) * bs + (ka % bs));
+        const bf16x4 vb = *(const bf16x4*)(p.vcache + (((size_t)pb * nkv + kvh) * hd + d) * bs + (kb % bs));
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          vf[dt][h][e] = va[e];
+          vf[dt][h][4 + e] = vb[e];
+        }
+      }
+    }
+    // ---- scale, cap, mask, running softmax (one query row per lane)
+    float mt = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int key = key0 + 8 * j + 4 * lk + i;
+        float v = s[4 * j + i] * p.scale;
+        if (p.softcap > 0.f) v = p.softcap * fast_tanh(v / p.softcap);
+        const bool ok = row_ok && key >= row_lo && key <= pos && key >= key_lo && key <= key_hi;
+        v = ok ? v : -INFINITY;
+        s[4 * j + i] = v;
+        mt = fmaxf(mt, v);
+      }
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m_run, mt);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = __expf(m_run - m_use);
+    float rs = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      const float pe = __expf(s[e] - m_use);
+      s[e] = pe;
+      rs += pe;
+    }
+    rs += __shfl_xor(rs, 32, 64);
+    l_run = l_run * corr + rs;
+    m_run = m_new;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) pb[h][e] = (__bf16)s[8 * h + e];
+    // ---- O^T = corr * O^T + V^T P^T
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+      for (int e = 0; e < 16; e++) o[dt][e] *= corr;
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][0], pb[0], o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][1], pb[1], o[dt], 0, 0, 0);
+    }
+  }
+  if (!row_ok) return;
+  if (SPLIT) {
+    const size_t slot = ((size_t)(r - p.r_begin) * p.nh + head) * p.nchunks + chunk;
+    if (lk == 0) {
+      p.part_ml[slot * 2] = m_run;
+      p.part_ml[slot * 2 + 1] = l_run;
+    }
+    float* po = p.part_o + slot * hd;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int d = dt * 32 + 8 * j + 4 * lk;
+        if (d < hd) *(f32x4*)(po + d) = f32x4{o[dt][4 * j], o[dt][4 * j + 1], o[dt][4 * j + 2], o[dt][4 * j + 3]};
+      }
+  } else {
+    const float inv = 1.f / l_run;
+    __bf16* orow = p.out + ((size_t)trow * p.nh + head) * hd;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int d = dt * 32 + 8 * j + 4 * lk;
+        if (d < hd) {
+          bf16x4 w;
+#pragma unroll
+          for (int i = 0; i < 4; i++) w[i] = (__bf16)(o[dt][4 * j + i] * inv);
+          *(bf16x4*)(orow + d) = w;
+        }
+      }
+  }
+}
+
+// Joins the chunks of a decoded token's attention, in chunk order.
+__global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restrict__ part_o,
+                                                          const float* __restrict__ part_ml,
+                                                          const int* __restrict__ q_start,
+                                                          const int* __restrict__ ctx_len,
+                                                          __bf16* __restrict__ out, int nh, int hd,
+                                                          int window, int r_begin, int nchunks) {
+  const int rr = blockIdx.x, head = blockIdx.y;
+  const int r = r_begin + rr;
+  const int n = q_start[r + 1] - q_start[r];
+  if (n <= 0) return;
+  const int pos = ctx_len[r] - 1;
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int c0 = lo / ATT_CHUNK, c1 = pos / ATT_CHUNK;
+  const size_t base = ((size_t)rr * nh + head) * nchunks;
+  float m = -INFINITY;
+  for (int c = c0; c <= c1; c++) m = fmaxf(m, part_ml[(base + c) * 2]);
+  float l = 0.f;
+  for (int c = c0; c <= c1; c++) l += part_ml[(base + c) * 2 + 1] * __expf(part_ml[(base + c) * 2] - m);
+  const float inv = 1.f / l;
+  __bf16* orow = out + ((size_t)q_start[r] * nh + head) * hd;
+  for (int d = threadIdx.x; d < hd; d += 64) {
+    float acc = 0.f;
+    for (int c = c0; c <= c1; c++) acc += part_o[(base + c) * hd + d] * __expf(part_ml[(base + c) * 2] - m);
+    orow[d] = (__bf16)(acc * inv);
+  }
+}
+
+template <bool SPLIT>
+static int launch_attn(const AttnParams& p, dim3 grid, hipStream_t s) {
+  switch (p.hd / 16) {
+    case 1: attn_mfma_kernel<1, SPLIT><<<grid, 256, 0, s>>>(p); break;
+    case 2: attn_mfma_kernel<2, SPLIT><<<grid, 256, 0, s>>>(p); break;
+    case 4: attn_mfma_kernel<4, SPLIT><<<grid, 256, 0, s>>>(p); break;
+    case 8: attn_mfma_kernel<8, SPLIT><<<grid, 256, 0, s>>>(p); break;
+    case 16: attn_mfma_kernel<16, SPLIT><<<grid, 256, 0, s>>>(p); break;
+    default: return zk_fail("zk_attention_bf16: head_dim must be 16, 32, 64, 128 or 256");
+  }
+  return zk_launch_status("zk_attention_bf16");
+}
+
+extern "C" {
+
+// 1 if the matrix-core kernel takes these sizes, else 0 (the caller then uses the plain kernel).
+int zk_attention_bf16_supports(int nh, int nkv, int hd, int bs) {
+  if (nkv <= 0 || nh % nkv) return 0;
+  const int g = nh / nkv;
+  const bool hd_ok = hd == 16 || hd == 32 || hd == 64 || hd == 128 || hd == 256;
+  return hd_ok && g <= 32 && bs % 4 == 0;
+}
+
+// Bytes of workspace the split variant needs for ``n_decode`` single-token requests.
+size_t zk_attention_bf16_workspace(int n_decode, int nh, int hd, int max_ctx) {
+  const size_t nchunks = ((size_t)max_ctx + ATT_CHUNK - 1) / ATT_CHUNK;
+  return (size_t)n_decode * nh * nchunks * (hd + 2) * sizeof(float);
+}
+
+// Requests [0, r_prefill) hold portions of more than one token (max_q_len the longest);
+// requests [r_prefill, R) hold one token each and use the split variant over max_ctx keys.
+int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const void* vcache_t,
+                      const int* block_table, int max_blocks, const int* q_start, const int* ctx_len,
+                      void* out, int R, int r_prefill, int max_q_len, int max_ctx, int nh, int nkv,
+                      int hd, int bs, float scale, float softcap, int window, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  ZK_REQUIRE(R >= 0 && r_prefill >= 0 && r_prefill <= R, "zk_attention_bf16: bad request counts");
+  ZK_REQUIRE(zk_attention_bf16_supports(nh, nkv, hd, bs), "zk_attention_bf16: sizes not supported "
+             "(head_dim 16/32/64/128/256, at most 32 heads a KV head, page size a multiple of 4)");
+  ZK_REQUIRE(q_stride >= nh * hd && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0),
+             "zk_attention_bf16: q rows must be 16-byte aligned");
+  ZK_REQUIRE(max_blocks > 0 && nkv <= 65535 && R <= 65535, "zk_attention_bf16: grid too large");
+  if (R == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  AttnParams p;
+  p.q = (const __bf16*)q; p.q_stride = q_stride;
+  p.kcache = (const __bf16*)kcache; p.vcache = (const __bf16*)vcache_t;
+  p.block_table = block_table; p.max_blocks = max_blocks;
+  p.q_start = q_start; p.ctx_len = ctx_len; p.out = (__bf16*)out;
+  p.nh = nh; p.nkv = nkv; p.hd = hd; p.bs = bs;
+  p.scale = scale; p.softcap = softcap; p.window = window;
+  const int g = nh / nkv;
+  if (r_prefill > 0) {
+    ZK_REQUIRE(max_q_len > 0, "zk_attention_bf16: max_q_len must be positive");
+    p.tpw = 32 / g; p.r_begin = 0; p.nchunks = 1; p.part_o = nullptr; p.part_ml = nullptr;
+    const int groups = (max_q_len + p.tpw - 1) / p.tpw;
+    dim3 grid((groups + 3) / 4, nkv, r_prefill);
+    int rc = launch_attn<false>(p, grid, s);
+    if (rc) return rc;
+  }
+  const int n_dec = R - r_prefill;
+  if (n_dec > 0) {
+    ZK_REQUIRE(max_ctx > 0, "zk_attention_bf16: max_ctx must be positive");
+    const int nchunks = (max_ctx + ATT_CHUNK - 1) / ATT_CHUNK;
+    ZK_REQUIRE(zk_attention_bf16_workspace(n_dec, nh, hd, max_ctx) <= workspace_bytes,
+               "zk_attention_bf16: workspace too small for the split partial results");
+    p.tpw = 1; p.r_begin = r_prefill; p.nchunks = nchunks;
+    p.part_o = (float*)workspace;
+    p.part_ml = (float*)workspace + (size_t)n_dec * nh * nchunks * hd;
+    dim3 grid((nchunks + 3) / 4, nkv, n_dec);
+    int rc = launch_attn<true>(p, grid, s);
+    if (rc) return rc;
+    dim3 cgrid(n_dec, nh);
+    attn_combine_kernel<<<cgrid, 64, 0, s>>>(p.part_o, p.part_ml, q_start, ctx_len, (__bf16*)out, nh, hd,
+                                             window, r_prefill, nchunks);
+    return zk_launch_status("zk_attention_bf16 (combine)");
+  }
+  return 0;
+}
+
+}  // extern "C"
+
+#endif  // ZSE_ACT_BF16

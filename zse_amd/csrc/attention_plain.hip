@@ -21,7 +21,7 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
     const act_t* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ req_of_token, const int* __restrict__ positions,
     act_t* __restrict__ out, int nh, int nkv, int hd, int bs, float scale, float softcap,
-    int window) {
+    int window, int v_transposed) {
   __shared__ float sq[AP_MAX_HD];
   __shared__ float sp[64];
   __shared__ int spage[64];
@@ -72,8 +72,11 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
         for (int jj = 0; jj < 64; jj++) {
           const int pg = spage[jj];
           if (pg < 0) continue;
-          const act_t* vr = vcache + (((size_t)pg * nkv + kvh) * bs + ((j0 + jj) % bs)) * hd;
-          a = fmaf(sp[jj], to_f32(vr[d]), a);
+          const size_t head_base = ((size_t)pg * nkv + kvh) * bs * hd;
+          const size_t off = (j0 + jj) % bs;
+          const act_t v = v_transposed ? vcache[head_base + (size_t)d * bs + off]
+                                       : vcache[head_base + off * hd + d];
+          a = fmaf(sp[jj], to_f32(v), a);
         }
         acc[c] = a;
       }
@@ -87,11 +90,13 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
   }
 }
 
-// softcap <= 0: no cap; window <= 0: every earlier key is visible.
+// softcap <= 0: no cap; window <= 0: every earlier key is visible.  v_transposed: V is
+// cached as [page][kv head][hd][bs] instead of [page][kv head][bs][hd].
 extern "C" int zk_attention_plain(const void* q, int q_stride, const void* kcache, const void* vcache,
                                   const int* block_table, int max_blocks, const int* req_of_token,
                                   const int* positions, void* out, int T, int nh, int nkv, int hd,
-                                  int bs, float scale, float softcap, int window, void* stream) {
+                                  int bs, float scale, float softcap, int window, int v_transposed,
+                                  void* stream) {
   ZK_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && bs > 0 && max_blocks > 0,
              "zk_attention_plain: bad sizes");
   ZK_REQUIRE(nh % nkv == 0, "zk_attention_plain: heads must be a multiple of kv heads");
@@ -102,6 +107,6 @@ extern "C" int zk_attention_plain(const void* q, int q_stride, const void* kcach
   dim3 grid(T, nh);
   attention_plain_kernel<<<grid, 64, 0, (hipStream_t)stream>>>(
       (const act_t*)q, q_stride, (const act_t*)kcache, (const act_t*)vcache, block_table, max_blocks,
-      req_of_token, positions, (act_t*)out, nh, nkv, hd, bs, scale, softcap, window);
+      req_of_token, positions, (act_t*)out, nh, nkv, hd, bs, scale, softcap, window, v_transposed);
   return zk_launch_status("zk_attention_plain");
 }

@@ -127,12 +127,13 @@ __global__ void softcap_kernel(float* __restrict__ z, size_t n, float cap) {
 
 // qkv: [T, (nh + 2 nkv) hd] rows of [q | k | v].  q is rotated in place; k is
 // rotated and stored, v is stored, at slot = page * bs + offset of the token
-// (slot < 0: nothing stored).  Cache layout per layer: [page][kv head][bs][hd].
+// (slot < 0: nothing stored).  Cache layout per layer: K [page][kv head][bs][hd];
+// V the same, or transposed [page][kv head][hd][bs] when v_transposed is set.
 __global__ void rope_cache_write_kernel(act_t* __restrict__ qkv, const int* __restrict__ positions,
                                         const int* __restrict__ slot_map,
                                         const float* __restrict__ inv_freq, int rotary_dim,
                                         act_t* __restrict__ kcache, act_t* __restrict__ vcache,
-                                        int nh, int nkv, int hd, int bs) {
+                                        int nh, int nkv, int hd, int bs, int v_transposed) {
   const int t = blockIdx.x;
   const int head = blockIdx.y;  // [0,nh): q; [nh, nh+nkv): k; [nh+nkv, nh+2nkv): v
   act_t* src = qkv + (size_t)t * (nh + 2 * nkv) * hd + (size_t)head * hd;
@@ -144,6 +145,11 @@ __global__ void rope_cache_write_kernel(act_t* __restrict__ qkv, const int* __re
     const int kvh = (head - nh) % nkv;
     act_t* base = head < nh + nkv ? kcache : vcache;
     const size_t page = slot / bs, off = slot % bs;
+    if (head >= nh + nkv && v_transposed) {
+      act_t* vt = vcache + (page * nkv + kvh) * (size_t)hd * bs + off;
+      for (int i = threadIdx.x; i < hd; i += blockDim.x) vt[(size_t)i * bs] = src[i];
+      return;
+    }
     dst = base + ((page * nkv + kvh) * bs + off) * hd;
   }
   if (head < nh + nkv) {
@@ -271,7 +277,7 @@ int zk_softcap(float* z, size_t n, float cap, void* stream) {
 
 int zk_rope_cache_write(void* qkv, const int* positions, const int* slot_map, const float* inv_freq,
                         int rotary_dim, void* kcache, void* vcache, int T, int nh, int nkv, int hd,
-                        int bs, void* stream) {
+                        int bs, int v_transposed, void* stream) {
   ZK_REQUIRE(T >= 0 && nh > 0 && nkv >= 0 && hd > 0 && bs > 0, "zk_rope_cache_write: bad sizes");
   ZK_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && rotary_dim % 2 == 0,
              "zk_rope_cache_write: rotary_dim must be even and at most head_dim");
@@ -281,7 +287,7 @@ int zk_rope_cache_write(void* qkv, const int* positions, const int* slot_map, co
   dim3 grid(T, nh + 2 * nkv);
   rope_cache_write_kernel<<<grid, 64, 0, (hipStream_t)stream>>>((act_t*)qkv, positions, slot_map, inv_freq,
                                                                 rotary_dim, (act_t*)kcache,
-                                                                (act_t*)vcache, nh, nkv, hd, bs);
+                                                                (act_t*)vcache, nh, nkv, hd, bs, v_transposed);
   return zk_launch_status("zk_rope_cache_write");
 }
 

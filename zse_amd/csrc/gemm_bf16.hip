@@ -1,0 +1,296 @@
+// bfloat16 matrix products on the matrix cores (MFMA), float accumulation:
+//   C[M,N] = A[M,K] * W[N,K]^T        (weights [out, in], both operands K-contiguous)
+//
+// Two kernels, chosen by M:
+//  * skinny (M <= 64, decode): the weight matrix is streamed once from HBM.  A
+//    block owns a strip of 16 weight rows; its four waves split K and each feeds
+//    16x16x32 MFMAs straight from global memory: a lane's 16-byte load is exactly
+//    its MFMA operand (row = lane % 16, eight k values at 8 * (lane / 16)), so no
+//    LDS staging is needed.  Partial sums of the four waves meet in LDS.
+//  * tile (M > 64, prefill): 128x128x64 block tiles staged through LDS, four waves
+//    of 64 lanes, each a 64x64 corner built from 32x32x16 MFMAs.
+// Epilogues: plain store (bf16 or float), soft cap on float output (LM head), and
+// the gated activation act(gate) * up over a [2I, K] weight whose first I rows are
+// the gate (the feed-forward's first product; the [T, 2I] intermediate never
+// reaches memory).
+//
+// The reference's products are scalar-FMA tiles and a one-warp-per-row GEMV
+// (orchestrator/kernels.py:1075-1126, 2077-2107), gate and up separate
+// (orchestrator/model_runner.py:1270-1275).
+#include "common.h"
+
+#if ZSE_ACT_BF16
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+enum { EPI_NONE = 0, EPI_SOFTCAP = 1, EPI_GELU_TANH = 2, EPI_SILU = 3 };
+
+__device__ __forceinline__ float epi_gelu_tanh(float g) {
+  const float k = 0.7978845608028654f;
+  return 0.5f * g * (1.0f + tanhf(k * (g + 0.044715f * g * g * g)));
+}
+__device__ __forceinline__ float epi_gate(float g, float u, int epi) {
+  return (epi == EPI_GELU_TANH ? epi_gelu_tanh(g) : g / (1.0f + expf(-g))) * u;
+}
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; i++) z[i] = (__bf16)0.f;
+  return z;
+}
+
+// ------------------------------------------------------------------ skinny
+// GATED: the block also streams the strip of "up" rows I + n and stores act(g)*u.
+template <int MT, bool GATED>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const __bf16* __restrict__ A, int lda,
+                                                          const __bf16* __restrict__ W,
+                                                          void* __restrict__ C, int ldc, int c_is_f32,
+                                                          int M, int N, int K, int epi, float cap) {
+  constexpr int NS = GATED ? 2 : 1;
+  __shared__ f32x4 red[3][NS][MT][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, kq = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int wrow = min(n0 + r, N - 1);
+  const __bf16* wp[NS];
+  wp[0] = W + (size_t)wrow * K + kq * 8;
+  if (GATED) wp[NS - 1] = W + (size_t)(N + wrow) * K + kq * 8;
+  const __bf16* ap[MT];
+  bool av[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) {
+    const int m = mt * 16 + r;
+    av[mt] = m < M;
+    ap[mt] = A + (size_t)min(m, M - 1) * lda + kq * 8;
+  }
+  f32x4 acc[NS][MT];
+#pragma unroll
+  for (int s = 0; s < NS; s++)
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) acc[s][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  constexpr int STEPS = (MT * NS >= 4) ? 4 : 8;   // 32-wide k steps a wave loads before it multiplies
+  constexpr int KB = STEPS * 32;
+  for (int k0 = wave * KB; k0 < K; k0 += 4 * KB) {
+    bf16x8 wf[NS][STEPS], af[MT][STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+      const int k = k0 + s * 32;
+      const bool in = k + kq * 8 < K;
+#pragma unroll
+      for (int g = 0; g < NS; g++) wf[g][s] = in ? *(const bf16x8*)(wp[g] + k) : zero8();
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) af[mt][s] = (in && av[mt]) ? *(const bf16x8*)(ap[mt] + k) : zero8();
+    }
+#pragma unroll
+    for (int s = 0; s < STEPS; s++)
+#pragma unroll
+      for (int g = 0; g < NS; g++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+          acc[g][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][s], af[mt][s], acc[g][mt], 0, 0, 0);
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int g = 0; g < NS; g++)
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) red[wave - 1][g][mt][lane] = acc[g][mt];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+  // lane holds rows n = n0 + 4*kq + i (i = 0..3) of column m = mt*16 + r
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) {
+    const int m = mt * 16 + r;
+    f32x4 v[NS];
+#pragma unroll
+    for (int g = 0; g < NS; g++) v[g] = acc[g][mt] + red[0][g][mt][lane] + red[1][g][mt][lane] + red[2][g][mt][lane];
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int n = n0 + 4 * kq + i;
+      if (n >= N) continue;
+      float x = v[0][i];
+      if (GATED) x = epi_gate(x, v[NS - 1][i], epi);
+      else if (epi == EPI_SOFTCAP) x = cap * tanhf(x / cap);
+      if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
+      else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ tile
+#define GT_BM 128
+#define GT_BN 128
+#define GT_BK 64
+#define GT_LD (GT_BK + 8)
+
+template <bool GATED>
+__global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict__ A, int lda,
+                                                        const __bf16* __restrict__ W,
+                                                        void* __restrict__ C, int ldc, int c_is_f32,
+                                                        int M, int N, int K, int epi, float cap,
+                                                        int tiles_m, int tiles_n) {
+  __shared__ __bf16 sA[GT_BM][GT_LD];
+  __shared__ __bf16 sB[GT_BN][GT_LD];
+  // blocks that share a weight tile run on one XCD (ids go round-robin over 8 XCDs)
+  int id = blockIdx.x;
+  const int total = tiles_m * tiles_n;
+  if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
+  const int tn = id / tiles_m, tm = id % tiles_m;
+  const int m0 = tm * GT_BM;
+  const int ncols = GATED ? GT_BN / 2 : GT_BN;       // output columns of the block
+  const int n0 = tn * ncols;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lr = lane & 31, lk = lane >> 5;
+
+  // each thread moves four 16-byte pieces of A and of B per k tile
+  const __bf16* ga[4];
+  const __bf16* gb[4];
+  int srow[4], scol[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int c = tid + i * 256;
+    srow[i] = c >> 3;
+    scol[i] = (c & 7) * 8;
+    const int am = min(m0 + srow[i], M - 1);
+    ga[i] = A + (size_t)am * lda + scol[i];
+    int bn;
+    if (GATED) bn = srow[i] < 64 ? min(n0 + srow[i], N - 1) : N + min(n0 + srow[i] - 64, N - 1);
+    else bn = min(n0 + srow[i], N - 1);
+    gb[i] = W + (size_t)bn * K + scol[i];
+  }
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+  bf16x8 ra[4], rb[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const bool in = scol[i] < K;
+    ra[i] = in ? *(const bf16x8*)(ga[i]) : zero8();
+    rb[i] = in ? *(const bf16x8*)(gb[i]) : zero8();
+  }
+  for (int k0 = 0; k0 < K; k0 += GT_BK) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      *(bf16x8*)(&sA[srow[i]][scol[i]]) = ra[i];
+      *(bf16x8*)(&sB[srow[i]][scol[i]]) = rb[i];
+    }
+    __syncthreads();
+    const int kn = k0 + GT_BK;
+    if (kn < K) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const bool in = kn + scol[i] < K;
+        ra[i] = in ? *(const bf16x8*)(ga[i] + kn) : zero8();
+        rb[i] = in ? *(const bf16x8*)(gb[i] + kn) : zero8();
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < GT_BK / 16; ks++) {
+      bf16x8 fa[2], fb[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) fa[i] = *(const bf16x8*)(&sA[wm * 64 + i * 32 + lr][ks * 16 + lk * 8]);
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const int brow = GATED ? j * 64 + wn * 32 : wn * 64 + j * 32;
+        fb[j] = *(const bf16x8*)(&sB[brow + lr][ks * 16 + lk * 8]);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+  }
+  // acc[i][j][4*b + e] is row 8*b + 4*lk + e of the 32x32 tile, column lr
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const int m = m0 + wm * 64 + i * 32 + 8 * b + 4 * lk + e;
+        if (m >= M) continue;
+        if (GATED) {
+          const int n = n0 + wn * 32 + lr;
+          if (n < N) {
+            const float x = epi_gate(acc[i][0][4 * b + e], acc[i][1][4 * b + e], epi);
+            if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
+            else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 2; j++) {
+            const int n = n0 + wn * 64 + j * 32 + lr;
+            if (n >= N) continue;
+            float x = acc[i][j][4 * b + e];
+            if (epi == EPI_SOFTCAP) x = cap * tanhf(x / cap);
+            if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
+            else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
+          }
+        }
+      }
+    }
+  }
+}
+
+template <bool GATED>
+static int launch_skinny(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M,
+                         int N, int K, int epi, float cap, hipStream_t s) {
+  const int mt = (M + 15) / 16;
+  dim3 grid((N + 15) / 16);
+#define ZK_SKINNY(MT_)                                                                          \
+  gemm_skinny_kernel<MT_, GATED><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, \
+                                                      ldc, c_is_f32, M, N, K, epi, cap)
+  if (mt == 1) ZK_SKINNY(1);
+  else if (mt == 2) ZK_SKINNY(2);
+  else if (mt == 3) ZK_SKINNY(3);
+  else ZK_SKINNY(4);
+#undef ZK_SKINNY
+  return zk_launch_status("zk_gemm_bf16 (skinny)");
+}
+
+// epi: 0 none, 1 soft cap (cap > 0), 2 gelu_tanh gate, 3 silu gate.  For the gated
+// epilogues W is [2N, K] (gate rows, then up rows) and C is [M, N].
+extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
+                            int M, int N, int K, int epi, float cap, void* stream) {
+  ZK_REQUIRE(M >= 0 && N > 0 && K > 0, "zk_gemm_bf16: bad sizes");
+  ZK_REQUIRE(K % 8 == 0 && lda % 8 == 0, "zk_gemm_bf16: K and lda must be multiples of 8");
+  ZK_REQUIRE(lda >= K && ldc >= N, "zk_gemm_bf16: leading dimensions too small");
+  ZK_REQUIRE(epi >= 0 && epi <= 3, "zk_gemm_bf16: unknown epilogue");
+  ZK_REQUIRE(epi != EPI_SOFTCAP || cap > 0.f, "zk_gemm_bf16: soft cap must be positive");
+  ZK_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "zk_gemm_bf16: operands must be 16-byte aligned");
+  if (M == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const bool gated = epi >= EPI_GELU_TANH;
+  if (M <= 64) {
+    return gated ? launch_skinny<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, s)
+                 : launch_skinny<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, s);
+  }
+  const int tiles_m = (M + GT_BM - 1) / GT_BM;
+  const int ncols = gated ? GT_BN / 2 : GT_BN;
+  const int tiles_n = (N + ncols - 1) / ncols;
+  ZK_REQUIRE((long long)tiles_m * tiles_n < 2147483647LL, "zk_gemm_bf16: too many tiles");
+  dim3 grid(tiles_m * tiles_n);
+  if (gated)
+    gemm_tile_kernel<true><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32,
+                                                M, N, K, epi, cap, tiles_m, tiles_n);
+  else
+    gemm_tile_kernel<false><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32,
+                                                 M, N, K, epi, cap, tiles_m, tiles_n);
+  return zk_launch_status("zk_gemm_bf16 (tile)");
+}
+
+#endif  // ZSE_ACT_BF16

@@ -16,7 +16,8 @@ class CallCache:
     need: object = None              # PagedKV | StateNeed | None
     group: Optional[int] = None      # cache group of a paged need
     k: Optional[Tensor] = None       # [pages, kv heads, page size, head dim]
-    v: Optional[Tensor] = None
+    v: Optional[Tensor] = None       # the same, or [pages, kv heads, head dim, page size]
+    v_transposed: bool = False
     state_offset: int = 0            # byte offset inside a request's state slot
     state_bytes: int = 0
 

@@ -110,6 +110,7 @@ class StepContext:
         self.groups: List[GroupView] = []
         self.max_q_len = 0
         self.max_ctx = 0
+        self.n_multi = 0             # requests [0, n_multi) of the batch bring more than one token
         self.entries: List[Tuple[object, int, int, int]] = []   # (req, slot, start, n) on the host
         self.state = None            # Tensor uint8-as-float32 words [max_seqs, slot_words] or None
         self.slot_bytes = 0
@@ -160,6 +161,11 @@ class StepRunner:
                 cc.group = gid_of[i]
                 shape = (num_pages, need.num_kv_heads, self.page_size, need.head_dim)
                 cc.k = rt.zeros(shape, self.dtype)
+                mixer = model.blocks[model.plan.order[i].layer].mixer
+                cc.v_transposed = bool(self.tuned and getattr(mixer, "wants_v_transposed", None) and
+                                       mixer.wants_v_transposed(self.k, self.dtype, self.page_size))
+                if cc.v_transposed:
+                    shape = (num_pages, need.num_kv_heads, need.head_dim, self.page_size)
                 cc.v = rt.zeros(shape, self.dtype)
             elif isinstance(need, StateNeed):
                 cc.state_offset = slot_bytes
@@ -236,11 +242,16 @@ class StepRunner:
         req_of_token[T:] = 0
         for sm in slot_maps:
             sm[T:] = -1
+        # requests that bring more than one token come first: the attention kernels
+        # treat the two kinds apart; logits still come back in the order of the entries
+        order = sorted(range(R), key=lambda i: len(entries[i].tokens) == 1)
+        n_multi = sum(1 for e in entries if len(e.tokens) > 1)
         t = 0
-        n_rows = 0
         host_entries = []
+        first_token = [0] * R
         max_q = max_ctx = 0
-        for r, e in enumerate(entries):
+        for r, i in enumerate(order):
+            e = entries[i]
             n = len(e.tokens)
             start = m.computed(e.req)
             tokens[t:t + n] = np.asarray(e.tokens, dtype=np.int32)
@@ -252,22 +263,26 @@ class StepRunner:
             for g in range(G):
                 slot_maps[g][t:t + n] = m.slot_mapping(e.req, g, start, n)
                 m.fill_table_row(e.req, g, tables[g][r])
-            for w in e.want:
-                if not (0 <= w < n):
-                    raise ValueError(f"request {e.req!r}: wanted place {w} is not among its {n} tokens")
-                logit_rows[n_rows] = t + w
-                n_rows += 1
+            first_token[i] = t
             host_entries.append((e.req, m.slot(e.req), start, n))
             max_q, max_ctx = max(max_q, n), max(max_ctx, start + n)
             t += n
+        n_rows = 0
+        for i, e in enumerate(entries):
+            for w in e.want:
+                if not (0 <= w < len(e.tokens)):
+                    raise ValueError(f"request {e.req!r}: wanted place {w} is not among its "
+                                     f"{len(e.tokens)} tokens")
+                logit_rows[n_rows] = first_token[i] + w
+                n_rows += 1
         q_start[R:] = T
         ctx_len[R:] = 0
         slot_of_req[R:] = 0
         for g in range(G):
             tables[g][R:] = -1
-        return off, cur, T, R, n_rows, host_entries, max_q, max_ctx
+        return off, cur, T, R, n_rows, host_entries, max_q, max_ctx, n_multi
 
-    def _context(self, off, T_pad, R_pad, host_entries, max_q, max_ctx) -> StepContext:
+    def _context(self, off, T_pad, R_pad, host_entries, max_q, max_ctx, n_multi) -> StepContext:
         ctx = StepContext(self)
         base = self.meta_dev.ptr
         p = lambda name: base + off[name] * 4
@@ -278,7 +293,7 @@ class StepRunner:
         ctx.groups = [GroupView(p(f"table{g}"), self.max_blocks, p(f"slot_map{g}"), self.page_size)
                       for g in range(len(self.manager.groups))]
         ctx.entries = host_entries
-        ctx.max_q_len, ctx.max_ctx = max_q, max_ctx
+        ctx.max_q_len, ctx.max_ctx, ctx.n_multi = max_q, max_ctx, n_multi
         ctx.state, ctx.slot_bytes = self.state, self.slot_bytes
         return ctx
 
@@ -318,11 +333,11 @@ class StepRunner:
                 raise OutOfPages(f"request {e.req!r} needs pages for {upto} tokens and the pool "
                                  f"cannot give them: {m.stats()}")
         self.rt.wait_event(self.meta_copied)     # the last step's copy has left the host buffer
-        off, words, T, R, n_rows, host_entries, max_q, max_ctx = self._pack(entries, T, R)
+        off, words, T, R, n_rows, host_entries, max_q, max_ctx, n_multi = self._pack(entries, T, R)
         self._ensure_logits(n_rows)
         self.rt.copy_h2d_async(self.meta_dev.ptr, self.meta_host.ptr, words * 4)
         self.rt.record(self.meta_copied)
-        ctx = self._context(off, T, R, host_entries, max_q, max_ctx)
+        ctx = self._context(off, T, R, host_entries, max_q, max_ctx, n_multi)
         self.arena.reset()
         self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, self.logits.rows(0, n_rows))
         for e in entries:

@@ -53,6 +53,12 @@ class PagedAttention(Part):
         s = self.spec
         return PagedKV(s.num_kv_heads, s.head_dim, s.window)
 
+    def wants_v_transposed(self, kernels, dtype: str, page_size: int) -> bool:
+        """The matrix-core kernel reads V as [page][kv head][hd][bs]."""
+        s = self.spec
+        return bool(dtype == BF16 and kernels.has("zk_attention_bf16") and
+                    kernels.zk_attention_bf16_supports(s.num_heads, s.num_kv_heads, s.head_dim, page_size))
+
     def forward(self, ctx, x: Tensor, cache) -> Tensor:
         s, k = self.spec, ctx.k
         T = x.shape[0]
@@ -69,19 +75,21 @@ class PagedAttention(Part):
             inv_freq, rotary_dim = tables[0].ptr, tables[1]
         k.zk_rope_cache_write(qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map,
                               inv_freq or None, rotary_dim, cache.k.ptr, cache.v.ptr, T, nh, n_store,
-                              hd, g.page_size, ctx.stream)
+                              hd, g.page_size, 1 if cache.v_transposed else 0, ctx.stream)
         o = ctx.alloc((T, nh * hd))
         cap = float(s.softcap) if s.softcap else 0.0
         win = int(s.window) if s.window else 0
-        if ctx.dtype == BF16 and ctx.tuned and k.has("zk_attention_bf16"):
+        if cache.v_transposed and ctx.tuned:
+            # the matrix-core kernel; requests with more than one token come first in the batch
             k.zk_attention_bf16(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
-                                ctx.req_of_token, ctx.positions, ctx.q_start, ctx.R, o.ptr, T, nh,
-                                nkv, hd, g.page_size, s.scale, cap, win, ctx.max_q_len, ctx.max_ctx,
+                                ctx.q_start, ctx.ctx_len, o.ptr, ctx.R, ctx.n_multi, ctx.max_q_len,
+                                ctx.max_ctx, nh, nkv, hd, g.page_size, s.scale, cap, win,
                                 ctx.workspace.ptr, ctx.workspace.nbytes, ctx.stream)
         else:
             k.zk_attention_plain(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table,
                                  g.max_blocks, ctx.req_of_token, ctx.positions, o.ptr, T, nh, nkv,
-                                 hd, g.page_size, s.scale, cap, win, ctx.stream)
+                                 hd, g.page_size, s.scale, cap, win, 1 if cache.v_transposed else 0,
+                                 ctx.stream)
         return linear(ctx, o, self.w_o, ctx.alloc((T, s.hidden_size)))
 
 

@@ -15,7 +15,7 @@ import numpy as np
 
 from ..runtime.device import BF16, F32, Tensor
 from .base import Part, TensorReq, register_part
-from .ops import linear
+from .ops import linear, tuned_gemm
 
 
 class Embedding(Part):
@@ -59,6 +59,8 @@ class LMHead(Part):
     def forward(self, ctx, x: Tensor, out: Tensor) -> Tensor:
         """x: normed rows [K, hidden]; out: float logits [K, vocab]."""
         s = self.spec
+        if s.softcap and tuned_gemm(ctx, s.hidden_size):
+            return linear(ctx, x, self.weight, out, epilogue="softcap", cap=float(s.softcap))
         linear(ctx, x, self.weight, out)
         if s.softcap:
             ctx.k.zk_softcap(out.ptr, out.numel, float(s.softcap), ctx.stream)

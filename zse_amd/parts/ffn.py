@@ -11,7 +11,7 @@ from typing import List
 
 from ..runtime.device import Tensor
 from .base import Part, TensorReq, register_part
-from .ops import linear
+from .ops import linear, tuned_gemm
 
 ACTIVATION_CODES = {"gelu_tanh": 0, "silu": 1}
 
@@ -37,6 +37,9 @@ class GatedMLP(Part):
     def forward(self, ctx, x: Tensor) -> Tensor:
         s = self.spec
         T, I = x.shape[0], s.intermediate_size
+        if tuned_gemm(ctx, s.hidden_size):
+            a = linear(ctx, x, self.w_gu, ctx.alloc((T, I)), epilogue=s.activation)
+            return linear(ctx, a, self.w_down, ctx.alloc((T, s.hidden_size)))
         gu = linear(ctx, x, self.w_gu, ctx.alloc((T, 2 * I)))
         a = ctx.alloc((T, I))
         ctx.k.zk_gated_act(gu.ptr, a.ptr, T, I, ACTIVATION_CODES[s.activation], ctx.stream)

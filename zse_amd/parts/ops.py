@@ -4,15 +4,31 @@ from __future__ import annotations
 from ..runtime.device import BF16, F32, Tensor
 
 
-def linear(ctx, x: Tensor, w: Tensor, out: Tensor) -> Tensor:
+EPILOGUES = {None: 0, "softcap": 1, "gelu_tanh": 2, "silu": 3}
+
+
+def tuned_gemm(ctx, K: int) -> bool:
+    """True when the matrix-core product serves this step (bf16, tuned kernels on,
+    rows of K values that are whole 16-byte pieces)."""
+    return ctx.dtype == BF16 and ctx.tuned and ctx.k.has("zk_gemm_bf16") and K % 8 == 0
+
+
+def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0.0) -> Tensor:
     """out[M, N] = x[M, K] @ w[N, K]^T with float accumulation.
 
     ``out`` may be float32 (logits) or the activation type.  In the 32-bit
     library only the plain product exists; the bf16 library picks a matrix-core
-    kernel by the number of rows.
+    kernel by the number of rows.  ``epilogue`` (matrix-core product only):
+    "softcap" applies cap * tanh(x / cap); "gelu_tanh" / "silu" take w as
+    [2N, K], gate rows first, and store act(gate) * up.
     """
     M, K = x.shape
+    gated = epilogue in ("gelu_tanh", "silu")
     N, K2 = w.shape
+    if gated:
+        N //= 2
+    if epilogue is not None and not tuned_gemm(ctx, K):
+        raise ValueError("linear: epilogues belong to the matrix-core product")
     if K != K2 or out.shape != (M, N):
         raise ValueError(f"linear: x {x.shape}, w {w.shape}, out {out.shape} do not fit")
     if x.dtype != ctx.dtype or w.dtype != ctx.dtype:
@@ -21,8 +37,9 @@ def linear(ctx, x: Tensor, w: Tensor, out: Tensor) -> Tensor:
         raise ValueError(f"linear: out must be float32 or {ctx.dtype}, got {out.dtype}")
     out_f32 = 1 if out.dtype == F32 else 0
     k = ctx.k
-    if ctx.dtype == BF16 and ctx.tuned and k.has("zk_gemm_bf16"):
-        k.zk_gemm_bf16(x.ptr, K, w.ptr, out.ptr, N, out_f32, M, N, K, ctx.stream)
+    if tuned_gemm(ctx, K):
+        k.zk_gemm_bf16(x.ptr, K, w.ptr, out.ptr, N, out_f32, M, N, K, EPILOGUES[epilogue], float(cap),
+                       ctx.stream)
     else:
         k.zk_gemm_plain(x.ptr, K, w.ptr, out.ptr, N, out_f32, M, N, K, ctx.stream)
     return out

@@ -27,7 +27,7 @@ PKG_LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "_l
 ARCH = "gfx950"
 
 COMMON_KERNELS = ["elementwise.hip", "gemm_plain.hip", "attention_plain.hip", "sampling.hip"]
-BF16_KERNELS = []
+BF16_KERNELS = ["gemm_bf16.hip", "attention_bf16.hip"]
 
 LIBRARIES: Dict[str, dict] = {
     "runtime": {"sources": ["runtime.cpp"], "defines": [], "device": False},

@@ -145,18 +145,22 @@ KERNEL_SIGNATURES = {
     "zk_norm_add_norm": [_VP, _VP, _F, _I, _VP, _VP, _F, _I, _VP, _I, _I, _VP],
     "zk_gated_act": [_VP, _VP, _I, _I, _I, _VP],
     "zk_softcap": [_VP, _SZ, _F, _VP],
-    "zk_rope_cache_write": [_VP, _VP, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "zk_rope_cache_write": [_VP, _VP, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
     "zk_convert": [_VP, _I, _VP, _I, _SZ, _VP],
     "zk_fill_normal": [_VP, _I, _SZ, _U64, _U64, _F, _F, _VP],
     "zk_zero": [_VP, _SZ, _VP],
     "zk_gemm_plain": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "zk_attention_plain": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _F,
-                           _I, _VP],
+                           _I, _I, _VP],
     "zk_argmax": [_VP, _VP, _I, _I, _VP],
     "zk_sample": [_VP, _VP, _VP, _VP, _VP, _I, _I, _VP],
 }
 # present only in the bf16 library
-BF16_KERNEL_SIGNATURES = {}
+BF16_KERNEL_SIGNATURES = {
+    "zk_gemm_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _VP],
+    "zk_attention_bf16": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
+                          _F, _F, _I, _VP, _SZ, _VP],
+}
 
 
 class KernelLibrary:
@@ -178,6 +182,13 @@ class KernelLibrary:
             fn.argtypes = args
             fn.restype = C.c_int
             setattr(self, name, self._wrap(name, fn))
+        if dtype == BF16:
+            self._dll.zk_attention_bf16_supports.restype = C.c_int
+            self._dll.zk_attention_bf16_supports.argtypes = [_I, _I, _I, _I]
+            self.zk_attention_bf16_supports = self._dll.zk_attention_bf16_supports
+            self._dll.zk_attention_bf16_workspace.restype = C.c_size_t
+            self._dll.zk_attention_bf16_workspace.argtypes = [_I, _I, _I, _I]
+            self.zk_attention_bf16_workspace = self._dll.zk_attention_bf16_workspace
         want = 1 if dtype == BF16 else 0
         if self._dll.zk_act_is_bf16() != want:
             raise DeviceError(f"{path} was built for the other storage type")
