@@ -151,3 +151,41 @@ def test_trace_run_program(cases, tmp_path):
         assert z.shape[0] == len(items)
         for row, (r, q) in zip(z, items):
             assert_close(row, refs[r][q], dtype, f"trace_run step {i} {r}@{q}")
+
+
+def test_graph_replays_match_eager_steps(cases):
+    """Decode steps through captured graphs, replayed many times with eager steps of other
+    shapes between them, against the same steps run without graphs."""
+    name, dtype = "B", "bfloat16"
+    folder, streams, refs = cases[(name, dtype)]
+    reqs = ["r0", "r2", "r5"]
+
+    def run(use_graphs):
+        runner = make_runner(folder, dtype, page_size=16, cache_tokens=512, max_seqs=4,
+                             max_batch_tokens=256, max_model_len=256, use_graphs=use_graphs)
+        fed = {r: 20 + 7 * i for i, r in enumerate(reqs)}
+        from zse_amd.engine.runner import StepEntry
+        for r in reqs:
+            runner.step([StepEntry(r, streams[r][:fed[r]], [])])
+        rows = {r: [] for r in reqs}
+        for step in range(14):
+            live = reqs if step % 5 != 4 else reqs[:2]           # the batch changes its bucket
+            z = runner.step([StepEntry(r, [streams[r][fed[r]]], [0]) for r in live])
+            for r, row in zip(live, z):
+                rows[r].append(row)
+                fed[r] += 1
+            if step % 3 == 1:                                      # eager work of another shape between replays
+                runner.step([StepEntry("other", streams["r4"][:9 + step], [0])])
+                runner.finish("other")
+        assert (len(runner.graphs) > 0) == use_graphs
+        if use_graphs:
+            assert any(isinstance(g, int) for g in runner.graphs.values())
+        return rows, fed
+
+    eager, fed = run(False)
+    graph, _ = run(True)
+    for i, r in enumerate(reqs):
+        got, want = np.stack(graph[r]), np.stack(eager[r])
+        assert np.array_equal(got, want), f"{r}: graph replay differs from the eager step"
+        start = 20 + 7 * i
+        assert_close(got, refs[r][start:start + len(got)], dtype, f"graph decode {r}")

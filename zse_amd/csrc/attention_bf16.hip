@@ -219,13 +219,17 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
   }
 }
 
-// Joins the chunks of a decoded token's attention, in chunk order.
-__global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restrict__ part_o,
-                                                          const float* __restrict__ part_ml,
-                                                          const int* __restrict__ q_start,
-                                                          const int* __restrict__ ctx_len,
-                                                          __bf16* __restrict__ out, int nh, int hd,
-                                                          int window, int r_begin, int nchunks) {
+// Joins the chunks of a decoded token's attention, in chunk order: a block per
+// (request, head), a thread per channel; the chunks' weights exp(m_c - m) are computed once.
+#define ATT_MAX_CHUNKS 1024
+__global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restrict__ part_o,
+                                                           const float* __restrict__ part_ml,
+                                                           const int* __restrict__ q_start,
+                                                           const int* __restrict__ ctx_len,
+                                                           __bf16* __restrict__ out, int nh, int hd,
+                                                           int window, int r_begin, int nchunks) {
+  __shared__ float wgt[ATT_MAX_CHUNKS];
+  __shared__ float red[17];
   const int rr = blockIdx.x, head = blockIdx.y;
   const int r = r_begin + rr;
   const int n = q_start[r + 1] - q_start[r];
@@ -235,14 +239,24 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
   const int c0 = lo / ATT_CHUNK, c1 = pos / ATT_CHUNK;
   const size_t base = ((size_t)rr * nh + head) * nchunks;
   float m = -INFINITY;
-  for (int c = c0; c <= c1; c++) m = fmaxf(m, part_ml[(base + c) * 2]);
+  for (int c = c0 + threadIdx.x; c <= c1; c += 256) m = fmaxf(m, part_ml[(base + c) * 2]);
+  m = wave_max(m);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
   float l = 0.f;
-  for (int c = c0; c <= c1; c++) l += part_ml[(base + c) * 2 + 1] * __expf(part_ml[(base + c) * 2] - m);
+  for (int c = c0 + threadIdx.x; c <= c1; c += 256) {
+    const float w = __expf(part_ml[(base + c) * 2] - m);
+    wgt[c - c0] = w;
+    l += part_ml[(base + c) * 2 + 1] * w;
+  }
+  l = block_sum(l, red);
   const float inv = 1.f / l;
   __bf16* orow = out + ((size_t)q_start[r] * nh + head) * hd;
-  for (int d = threadIdx.x; d < hd; d += 64) {
+  for (int d = threadIdx.x; d < hd; d += 256) {
     float acc = 0.f;
-    for (int c = c0; c <= c1; c++) acc += part_o[(base + c) * hd + d] * __expf(part_ml[(base + c) * 2] - m);
+    for (int c = c0; c <= c1; c++) acc += part_o[(base + c) * hd + d] * wgt[c - c0];
     orow[d] = (__bf16)(acc * inv);
   }
 }
@@ -319,8 +333,9 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
     dim3 grid((nchunks + 3) / 4, nkv, n_dec);
     int rc = launch_attn<true>(p, grid, s);
     if (rc) return rc;
+    ZK_REQUIRE(nchunks <= ATT_MAX_CHUNKS, "zk_attention_bf16: context too long for the split variant");
     dim3 cgrid(n_dec, nh);
-    attn_combine_kernel<<<cgrid, 64, 0, s>>>(p.part_o, p.part_ml, q_start, ctx_len, (__bf16*)out, nh, hd,
+    attn_combine_kernel<<<cgrid, 256, 0, s>>>(p.part_o, p.part_ml, q_start, ctx_len, (__bf16*)out, nh, hd,
                                              window, r_prefill, nchunks);
     return zk_launch_status("zk_attention_bf16 (combine)");
   }

@@ -98,6 +98,132 @@ __global__ void norm_add_norm_kernel(const act_t* __restrict__ sub, const float*
     o[i] = from_f32<act_t>(hr[i] * rs2 * gain(w_next, i, uo_next));
 }
 
+// Single-pass variants for rows of up to 8192 values in whole groups of four: a
+// thread keeps its part of the row in registers (four values at tid*4 + j*1024), so the
+// row is read once and the two block sums are the only synchronisation.
+#define NF_MAXV 8
+
+template <typename TIn>
+__device__ __forceinline__ void load4(const TIn* p, float v[4]);
+template <>
+__device__ __forceinline__ void load4<float>(const float* p, float v[4]) {
+  const float4 t = *(const float4*)p;
+  v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+template <>
+__device__ __forceinline__ void load4<__bf16>(const __bf16* p, float v[4]) {
+  typedef __bf16 b4 __attribute__((ext_vector_type(4)));
+  const b4 t = *(const b4*)p;
+#pragma unroll
+  for (int i = 0; i < 4; i++) v[i] = (float)t[i];
+}
+__device__ __forceinline__ void store4(float* p, const float v[4]) {
+  *(float4*)p = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store4(__bf16* p, const float v[4]) {
+  typedef __bf16 b4 __attribute__((ext_vector_type(4)));
+  b4 t;
+#pragma unroll
+  for (int i = 0; i < 4; i++) t[i] = (__bf16)v[i];
+  *(b4*)p = t;
+}
+
+template <typename TIn>
+__global__ __launch_bounds__(256) void rmsnorm_fast_kernel(const TIn* __restrict__ x,
+                                                           const int* __restrict__ rows,
+                                                           const float* __restrict__ w,
+                                                           act_t* __restrict__ out, float eps,
+                                                           int unit_offset, int H) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const TIn* xr = x + (size_t)(rows ? rows[r] : r) * H;
+  float v[NF_MAXV][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NF_MAXV; j++) {
+    const int i = threadIdx.x * 4 + j * 1024;
+    if (i < H) {
+      load4<TIn>(xr + i, v[j]);
+#pragma unroll
+      for (int e = 0; e < 4; e++) ss += v[j][e] * v[j][e];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float rs = rsqrtf(ss / (float)H + eps);
+  act_t* o = out + (size_t)r * H;
+#pragma unroll
+  for (int j = 0; j < NF_MAXV; j++) {
+    const int i = threadIdx.x * 4 + j * 1024;
+    if (i < H) {
+      float g[4], y[4];
+      load4<float>(w + i, g);
+#pragma unroll
+      for (int e = 0; e < 4; e++) y[e] = v[j][e] * rs * (unit_offset ? 1.f + g[e] : g[e]);
+      store4(o + i, y);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
+    const act_t* __restrict__ sub, const float* __restrict__ w_post, float eps_post, int uo_post,
+    float* __restrict__ h, const float* __restrict__ w_next, float eps_next, int uo_next,
+    act_t* __restrict__ out, int H) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const act_t* s = sub + (size_t)r * H;
+  float* hr = h + (size_t)r * H;
+  float v[NF_MAXV][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NF_MAXV; j++) {
+    const int i = threadIdx.x * 4 + j * 1024;
+    if (i < H) {
+      load4<act_t>(s + i, v[j]);
+#pragma unroll
+      for (int e = 0; e < 4; e++) ss += v[j][e] * v[j][e];
+    }
+  }
+  float rs = 1.f;
+  if (w_post) {
+    ss = block_sum(ss, red);
+    rs = rsqrtf(ss / (float)H + eps_post);
+  }
+  float ss2 = 0.f;
+#pragma unroll
+  for (int j = 0; j < NF_MAXV; j++) {
+    const int i = threadIdx.x * 4 + j * 1024;
+    if (i < H) {
+      float g[4], hv[4];
+      load4<float>(hr + i, hv);
+      if (w_post) load4<float>(w_post + i, g);
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        float t = v[j][e];
+        if (w_post) t = t * rs * (uo_post ? 1.f + g[e] : g[e]);
+        t = hv[e] + t;
+        v[j][e] = t;
+        ss2 += t * t;
+      }
+      store4(hr + i, v[j]);
+    }
+  }
+  if (!w_next) return;
+  ss2 = block_sum(ss2, red);
+  const float rs2 = rsqrtf(ss2 / (float)H + eps_next);
+  act_t* o = out + (size_t)r * H;
+#pragma unroll
+  for (int j = 0; j < NF_MAXV; j++) {
+    const int i = threadIdx.x * 4 + j * 1024;
+    if (i < H) {
+      float g[4], y[4];
+      load4<float>(w_next + i, g);
+#pragma unroll
+      for (int e = 0; e < 4; e++) y[e] = v[j][e] * rs2 * (uo_next ? 1.f + g[e] : g[e]);
+      store4(o + i, y);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ gated activation
 
 __device__ __forceinline__ float gelu_tanh(float g) {
@@ -239,6 +365,13 @@ int zk_rmsnorm(const void* x, int x_is_f32, const int* rows, const float* w, voi
   ZK_REQUIRE(R >= 0 && H > 0, "zk_rmsnorm: bad sizes");
   if (R == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  if (H % 4 == 0 && H <= NF_MAXV * 1024) {
+    if (x_is_f32)
+      rmsnorm_fast_kernel<float><<<R, 256, 0, s>>>((const float*)x, rows, w, (act_t*)out, eps, unit_offset, H);
+    else
+      rmsnorm_fast_kernel<act_t><<<R, 256, 0, s>>>((const act_t*)x, rows, w, (act_t*)out, eps, unit_offset, H);
+    return zk_launch_status("zk_rmsnorm");
+  }
   if (x_is_f32)
     rmsnorm_kernel<float><<<R, 256, 0, s>>>((const float*)x, rows, w, (act_t*)out, eps, unit_offset, H);
   else
@@ -252,6 +385,12 @@ int zk_norm_add_norm(const void* sub, const float* w_post, float eps_post, int u
   ZK_REQUIRE(T >= 0 && H > 0, "zk_norm_add_norm: bad sizes");
   ZK_REQUIRE(w_next == nullptr || out != nullptr, "zk_norm_add_norm: next norm without output");
   if (T == 0) return 0;
+  if (H % 4 == 0 && H <= NF_MAXV * 1024) {
+    norm_add_norm_fast_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)sub, w_post, eps_post, uo_post,
+                                                                  h, w_next, eps_next, uo_next,
+                                                                  (act_t*)out, H);
+    return zk_launch_status("zk_norm_add_norm");
+  }
   norm_add_norm_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)sub, w_post, eps_post, uo_post, h,
                                                            w_next, eps_next, uo_next, (act_t*)out, H);
   return zk_launch_status("zk_norm_add_norm");

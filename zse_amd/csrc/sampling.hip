@@ -11,20 +11,10 @@
 // top-p cut-offs computed by the caller).
 #include "common.h"
 
-__global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ logits, int V,
-                                                     int* __restrict__ out) {
-  __shared__ float sv[256];
-  __shared__ int si[256];
-  const float* z = logits + (size_t)blockIdx.x * V;
-  float best = -INFINITY;
-  int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += 256) {
-    const float v = z[i];
-    if (v > best || (bi == 0x7fffffff && !(v != v))) {
-      best = v;
-      bi = i;
-    }
-  }
+// Stage 1: block (slice, row) scans its slice of the row; stage 2: one block a row joins the
+// slices.  Larger value wins, equal values go to the lower index, NaNs never win.
+#define AM_SLICES 64
+__device__ __forceinline__ void argmax_block_reduce(float& best, int& bi, float* sv, int* si) {
   sv[threadIdx.x] = best;
   si[threadIdx.x] = bi;
   __syncthreads();
@@ -39,7 +29,48 @@ __global__ __launch_bounds__(256) void argmax_kernel(const float* __restrict__ l
     }
     __syncthreads();
   }
-  if (threadIdx.x == 0) out[blockIdx.x] = si[0] == 0x7fffffff ? 0 : si[0];
+  best = sv[0];
+  bi = si[0];
+}
+
+__global__ __launch_bounds__(256) void argmax_slices_kernel(const float* __restrict__ logits, int V,
+                                                            float* __restrict__ pv, int* __restrict__ pi) {
+  __shared__ float sv[256];
+  __shared__ int si[256];
+  const int row = blockIdx.y, slice = blockIdx.x;
+  const float* z = logits + (size_t)row * V;
+  const int per = (V + AM_SLICES - 1) / AM_SLICES;
+  const int b = slice * per, e = min(V, b + per);
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = b + threadIdx.x; i < e; i += 256) {
+    const float v = z[i];
+    if (v > best || (bi == 0x7fffffff && v == v)) {
+      best = v;
+      bi = i;
+    }
+  }
+  argmax_block_reduce(best, bi, sv, si);
+  if (threadIdx.x == 0) {
+    pv[row * AM_SLICES + slice] = best;
+    pi[row * AM_SLICES + slice] = bi;
+  }
+}
+
+__global__ __launch_bounds__(256) void argmax_join_kernel(const float* __restrict__ pv,
+                                                          const int* __restrict__ pi,
+                                                          int* __restrict__ out) {
+  __shared__ float sv[256];
+  __shared__ int si[256];
+  const int row = blockIdx.x;
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  if (threadIdx.x < AM_SLICES) {
+    best = pv[row * AM_SLICES + threadIdx.x];
+    bi = pi[row * AM_SLICES + threadIdx.x];
+  }
+  argmax_block_reduce(best, bi, sv, si);
+  if (threadIdx.x == 0) out[row] = bi == 0x7fffffff ? 0 : bi;
 }
 
 // One block per row.  Thread i owns the contiguous segment [i*seg, (i+1)*seg).
@@ -120,10 +151,19 @@ __global__ __launch_bounds__(256) void sample_kernel(const float* __restrict__ l
 
 extern "C" {
 
-int zk_argmax(const float* logits, int* out, int rows, int V, void* stream) {
+// scratch: room for rows * 64 floats and rows * 64 ints (zk_argmax_scratch_bytes)
+size_t zk_argmax_scratch_bytes(int rows) { return (size_t)rows * AM_SLICES * 8; }
+
+int zk_argmax(const float* logits, int* out, int rows, int V, void* scratch, void* stream) {
   ZK_REQUIRE(rows >= 0 && V > 0, "zk_argmax: bad sizes");
+  ZK_REQUIRE(rows <= 65535, "zk_argmax: too many rows");
+  ZK_REQUIRE(scratch != nullptr, "zk_argmax: no scratch buffer");
   if (rows == 0) return 0;
-  argmax_kernel<<<rows, 256, 0, (hipStream_t)stream>>>(logits, V, out);
+  float* pv = (float*)scratch;
+  int* pi = (int*)scratch + (size_t)rows * AM_SLICES;
+  dim3 grid(AM_SLICES, rows);
+  argmax_slices_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(logits, V, pv, pi);
+  argmax_join_kernel<<<rows, 256, 0, (hipStream_t)stream>>>(pv, pi, out);
   return zk_launch_status("zk_argmax");
 }
 

@@ -69,9 +69,24 @@ class Model:
         """Run the step's tokens through every entry of the order; write float
         logits of the rows ``logit_rows`` (device int32 pointer) into ``logits``."""
         h = self.embedding.forward(ctx)
-        for i, call in enumerate(self.plan.order):
+        order = self.plan.order
+        # the norm that opens a layer is computed by the kernel that closes the one before;
+        # its output alternates between two buffers that outlive a layer's own
+        T, H = h.shape
+        handoff = [ctx.alloc((T, H)), ctx.alloc((T, H))]
+        x = None
+        base = ctx.arena.mark()
+        for i, call in enumerate(order):
             cache = caches[call.cache_of if call.cache_of is not None else i]
-            self.blocks[call.layer].forward(ctx, h, cache)
+            blk = self.blocks[call.layer]
+            nxt = self.blocks[order[i + 1].layer] if i + 1 < len(order) else None
+            if hasattr(blk, "entry_norm"):
+                next_norm = nxt.entry_norm() if nxt is not None and hasattr(nxt, "entry_norm") else None
+                x = blk.forward(ctx, h, cache, x_in=x, next_norm=next_norm, x_out=handoff[i % 2])
+            else:
+                blk.forward(ctx, h, cache)
+                x = None
+            ctx.arena.release(base)
         if n_rows:
             x = self.final_norm.forward(ctx, h, out_rows=(logit_rows, n_rows))
             self.head.forward(ctx, x, logits)

@@ -187,7 +187,8 @@ class StepRunner:
         self.meta_copied = rt.event()
         rt.record(self.meta_copied)
         self.logits: Optional[Tensor] = None
-        self.graphs: Dict[int, dict] = {}
+        self.graphs: Dict[int, object] = {}      # bucket -> "warm" | graph handle
+        self.graph_logits: Optional[Tensor] = None
         self.steps_run = 0
 
     # ------------------------------------------------------------------ sizes
@@ -303,6 +304,57 @@ class StepRunner:
             self.logits = None
             self.logits = self.rt.empty((max(rows, 8), self.vocab), F32)
 
+    # ------------------------------------------------------------------ graphs for decode steps
+    def _graph_bucket(self, entries) -> int:
+        """The padded batch size under which a decode-only step replays a captured graph
+        (0: run eagerly).  Every entry brings one token and wants its logits."""
+        if not self.use_graphs or self.state is not None:
+            return 0
+        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
+            return 0
+        b = 1
+        while b < len(entries):
+            b *= 2
+        return b if b <= self.max_seqs else 0
+
+    def _graph_step(self, entries, bucket: int):
+        """One token for each request through the graph of this bucket.  The first step of
+        a bucket runs eagerly (it sizes the arena), the second is captured, later ones
+        replay.  Kernel arguments are fixed by the bucket: rows beyond the batch are
+        padding (position -1, no cache slot, no request), attention covers the longest
+        context the runner allows, and the logits land in a buffer of the graphs' own."""
+        R = len(entries)
+        off, words, T, _, n_rows, host_entries, _, _, _ = self._pack(entries, bucket, bucket)
+        logit_rows = self.meta_host.array(off["logit_rows"] * 4, bucket, np.int32)
+        logit_rows[n_rows:] = 0
+        self.rt.copy_h2d_async(self.meta_dev.ptr, self.meta_host.ptr, words * 4)
+        self.rt.record(self.meta_copied)
+        if self.graph_logits is None:
+            self.graph_logits = self.rt.empty((self.max_seqs, self.vocab), F32)
+        out = self.graph_logits.rows(0, bucket)
+        state = self.graphs.get(bucket)
+        if isinstance(state, int):
+            self.rt.graph_launch(state)
+            return self.graph_logits.rows(0, n_rows)
+        ctx = self._context(off, bucket, bucket, host_entries, 1, self.max_model_len, 0)
+        self.arena.reset()
+        if state is None:                       # first time: eager, lets the arena grow
+            self.model.forward(ctx, self.caches, ctx.logit_rows, bucket, out)
+            self.graphs[bucket] = "warm"
+            return self.graph_logits.rows(0, n_rows)
+        self.arena.frozen = True
+        try:
+            self.rt.capture_begin()
+            try:
+                self.model.forward(ctx, self.caches, ctx.logit_rows, bucket, out)
+            finally:
+                graph = self.rt.capture_end()
+        finally:
+            self.arena.frozen = False
+        self.graphs[bucket] = graph
+        self.rt.graph_launch(graph)
+        return self.graph_logits.rows(0, n_rows)
+
     def step(self, entries: Sequence[StepEntry], download: bool = True):
         """Run one step.  Returns float32 logits [wanted, vocab] on the host
         (``download=False``: the device tensor, valid until the next step)."""
@@ -333,17 +385,21 @@ class StepRunner:
                 raise OutOfPages(f"request {e.req!r} needs pages for {upto} tokens and the pool "
                                  f"cannot give them: {m.stats()}")
         self.rt.wait_event(self.meta_copied)     # the last step's copy has left the host buffer
-        off, words, T, R, n_rows, host_entries, max_q, max_ctx, n_multi = self._pack(entries, T, R)
-        self._ensure_logits(n_rows)
-        self.rt.copy_h2d_async(self.meta_dev.ptr, self.meta_host.ptr, words * 4)
-        self.rt.record(self.meta_copied)
-        ctx = self._context(off, T, R, host_entries, max_q, max_ctx, n_multi)
-        self.arena.reset()
-        self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, self.logits.rows(0, n_rows))
+        bucket = self._graph_bucket(entries)
+        if bucket:
+            out = self._graph_step(entries, bucket)
+        else:
+            off, words, T, R, n_rows, host_entries, max_q, max_ctx, n_multi = self._pack(entries, T, R)
+            self._ensure_logits(n_rows)
+            self.rt.copy_h2d_async(self.meta_dev.ptr, self.meta_host.ptr, words * 4)
+            self.rt.record(self.meta_copied)
+            ctx = self._context(off, T, R, host_entries, max_q, max_ctx, n_multi)
+            self.arena.reset()
+            out = self.logits.rows(0, n_rows)
+            self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, out)
         for e in entries:
             m.commit(e.req, m.computed(e.req) + len(e.tokens))
         self.steps_run += 1
-        out = self.logits.rows(0, n_rows)
         if not download:
             return out
         return self.rt.download(out)

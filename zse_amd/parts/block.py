@@ -32,14 +32,18 @@ class Block(Part):
     def children(self):
         return list(self.norms.values()) + [self.mixer, self.ffn]
 
-    def _join(self, ctx, sub: Tensor, post, h: Tensor, nxt):
-        """h += post(sub) (post None: h += sub); returns nxt(h) if nxt is given."""
+    def _join(self, ctx, sub: Tensor, post, h: Tensor, nxt, out: Tensor = None):
+        """h += post(sub) (post None: h += sub); returns nxt(h) if nxt is given, written
+        to ``out`` when the caller brings a buffer."""
         T, H = h.shape
         fused_post = post is None or isinstance(post, RMSNorm)
         fused_next = nxt is None or isinstance(nxt, RMSNorm)
         if not fused_post:
             sub, post = post.forward(ctx, sub), None
-        out = ctx.alloc((T, H)) if (nxt is not None and fused_next) else None
+        if nxt is None or not fused_next:
+            out = None
+        elif out is None:
+            out = ctx.alloc((T, H))
         ps = post.spec if post is not None else None
         ns = nxt.spec if (nxt is not None and fused_next) else None
         ctx.k.zk_norm_add_norm(
@@ -51,15 +55,24 @@ class Block(Part):
             out = nxt.forward(ctx, h)
         return out
 
-    def forward(self, ctx, h: Tensor, cache) -> None:
+    def entry_norm(self):
+        """The norm this block applies to the stream first; the block before may apply it
+        for us in the kernel that ends its own work (see ``forward``)."""
+        return self.norms["pre_mixer"]
+
+    def forward(self, ctx, h: Tensor, cache, x_in: Tensor = None, next_norm=None, x_out: Tensor = None):
+        """Update the stream ``h`` in place.  ``x_in``: this block's entry norm of ``h``,
+        if the caller already has it.  ``next_norm``: the entry norm of whatever runs
+        next; its output is returned (computed in the same kernel as the last
+        residual sum), in ``x_out`` if given."""
         n = self.norms
-        mark = ctx.arena.mark()
-        x = n["pre_mixer"].forward(ctx, h)
+        x = x_in if x_in is not None else n["pre_mixer"].forward(ctx, h)
         a = self.mixer.forward(ctx, x, cache)
         x = self._join(ctx, a, n.get("post_mixer"), h, n["pre_ffn"])
         m = self.ffn.forward(ctx, x)
-        self._join(ctx, m, n.get("post_ffn"), h, None)
-        ctx.arena.release(mark)
+        if not isinstance(next_norm, RMSNorm):
+            next_norm = None         # a norm the closing kernel does not know: the next block applies it
+        return self._join(ctx, m, n.get("post_ffn"), h, next_norm, x_out)
 
 
 register_part("block", "block", Block)

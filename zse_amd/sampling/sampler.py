@@ -123,6 +123,7 @@ class DeviceSampler:
         self.ids2 = rt.empty((max_rows,), I32)
         self.temp = rt.empty((max_rows,), F32)
         self.u = rt.empty((max_rows,), F64)
+        self.scratch = rt.empty((max_rows * 128,), F32)     # slices of the two-stage argmax
 
     def sample(self, logits, rows: Sequence[dict]) -> List[int]:
         """``logits``: device float32 [n, vocab]; ``rows``: per row a dict with
@@ -138,7 +139,7 @@ class DeviceSampler:
         need_host = [i for i, r in enumerate(rows) if not r["params"].on_device]
         out: List[Optional[int]] = [None] * n
         if need_greedy:
-            k.zk_argmax(logits.ptr, self.ids.ptr, n, V, rt.stream)
+            k.zk_argmax(logits.ptr, self.ids.ptr, n, V, self.scratch.ptr, rt.stream)
         if need_temp:
             t = np.array([r["params"].temperature if not r["params"].greedy else 1.0 for r in rows],
                          dtype=np.float32)
