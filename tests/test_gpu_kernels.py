@@ -25,6 +25,22 @@ def up(rt, x, dtype):
     return rt.upload(f32_to_bf16_bits(x), "bfloat16") if dtype == "bfloat16" else rt.upload(x, "float32")
 
 
+_ALIVE = []
+
+
+@pytest.fixture(autouse=True)
+def _drop_device_tensors():
+    yield
+    _ALIVE.clear()
+
+
+def ptr(t):
+    """A tensor's device pointer; the tensor stays allocated until the test ends (a kernel
+    that was only enqueued must not find its operand freed)."""
+    _ALIVE.append(t)
+    return t.ptr
+
+
 def gelu(z):
     return 0.5 * z * (1 + np.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
 
@@ -213,3 +229,200 @@ def test_attention_over_pages(rt, kernel, case):
     tol = 2e-5 if dtype == "float32" else 0.02
     err = np.abs(got - want)
     assert err.max() < tol, f"max error {err.max()} at token {np.unravel_index(err.argmax(), err.shape)}"
+
+
+# ------------------------------------------------------------------ row-wise kernels
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T,H,V", [(5, 96, 1000), (3, 2304, 300), (1, 70, 17)])
+def test_embed(rt, dtype, T, H, V):
+    k = rt.kernels(dtype)
+    rng = np.random.default_rng(T + H)
+    table = rng.normal(size=(V, H)).astype(np.float32)
+    if dtype == "bfloat16":
+        table = bf16(table)
+    toks = rng.integers(0, V, T).astype(np.int32)
+    toks[0] = V - 1
+    out = rt.empty((T, H), "float32")
+    k.zk_embed(ptr(up(rt, table, dtype)), ptr(rt.upload(toks)), out.ptr, 9.8125, T, H, V, rt.stream)
+    assert np.array_equal(rt.download(out), table[toks] * np.float32(9.8125))      # (ref) rows of the table
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T,H,eps,uo", [(4, 96, 1e-5, 1), (3, 2304, 1e-6, 1), (2, 70, 1e-6, 0), (2, 9000, 1e-6, 1)])
+def test_rmsnorm_and_the_fused_joins(rt, dtype, T, H, eps, uo):
+    k = rt.kernels(dtype)
+    rng = np.random.default_rng(H)
+    tol = 1e-5 if dtype == "float32" else 2.0 ** -7
+    x = rng.normal(size=(T, H)).astype(np.float32) * 3
+    w = rng.normal(size=H).astype(np.float32) * 0.3
+    w2 = rng.normal(size=H).astype(np.float32) * 0.3
+    gain = lambda v: (1 + v) if uo else v
+    norm = lambda a, v: a / np.sqrt((a * a).mean(-1, keepdims=True) + eps) * gain(v)
+    W, W2 = rt.upload(w), rt.upload(w2)
+    out = rt.empty((T, H), dtype)
+    k.zk_rmsnorm(ptr(rt.upload(x)), 1, None, W.ptr, out.ptr, eps, uo, T, H, rt.stream)
+    want = norm(x.astype(np.float64), w)
+    assert np.abs(rt.download_f32(out) - want).max() <= tol * np.abs(want).max()
+    # rows picked by index
+    rows = np.array([T - 1, 0], np.int32)
+    out2 = rt.empty((2, H), dtype)
+    k.zk_rmsnorm(ptr(rt.upload(x)), 1, ptr(rt.upload(rows)), W.ptr, out2.ptr, eps, uo, 2, H, rt.stream)
+    assert np.abs(rt.download_f32(out2) - want[rows]).max() <= tol * np.abs(want).max()
+    # (ref) all ones with unit gain come out as ones
+    ones = rt.empty((1, H), dtype)
+    k.zk_rmsnorm(ptr(rt.upload(np.ones((1, H), np.float32))), 1, None, ptr(rt.upload(np.zeros(H, np.float32))),
+                 ones.ptr, 1e-6, 1, 1, H, rt.stream)
+    assert np.abs(rt.download_f32(ones) - 1.0).max() < 1e-3
+    # h += N_post(sub); out = N_next(h)
+    sub = rng.normal(size=(T, H)).astype(np.float32)
+    if dtype == "bfloat16":
+        sub = bf16(sub)
+    h = rng.normal(size=(T, H)).astype(np.float32)
+    Hd = rt.upload(h)
+    nxt = rt.empty((T, H), dtype)
+    k.zk_norm_add_norm(ptr(up(rt, sub, dtype)), W.ptr, eps, uo, Hd.ptr, W2.ptr, eps * 2, uo, nxt.ptr, T, H, rt.stream)
+    h_want = h.astype(np.float64) + norm(sub.astype(np.float64), w)
+    assert np.abs(rt.download(Hd) - h_want).max() < 1e-5 * max(1, np.abs(h_want).max())     # the stream stays float
+    x_want = h_want / np.sqrt((h_want * h_want).mean(-1, keepdims=True) + eps * 2) * gain(w2)
+    assert np.abs(rt.download_f32(nxt) - x_want).max() <= tol * np.abs(x_want).max()
+    # no post norm: a plain residual sum; no next norm: nothing else is written
+    Hd2 = rt.upload(h)
+    k.zk_norm_add_norm(ptr(up(rt, sub, dtype)), None, 0.0, 0, Hd2.ptr, None, 0.0, 0, None, T, H, rt.stream)
+    assert np.abs(rt.download(Hd2) - (h.astype(np.float64) + sub)).max() < 1e-6
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gated_activation_and_softcap(rt, dtype):
+    k = rt.kernels(dtype)
+    rng = np.random.default_rng(3)
+    T, I = 3, 330
+    gu = rng.normal(size=(T, 2 * I)).astype(np.float32) * 2
+    if dtype == "bfloat16":
+        gu = bf16(gu)
+    g, u = gu[:, :I].astype(np.float64), gu[:, I:].astype(np.float64)
+    tol = 1e-5 if dtype == "float32" else 2.0 ** -7
+    for act, want in ((0, gelu(g) * u), (1, g / (1 + np.exp(-g)) * u)):
+        out = rt.empty((T, I), dtype)
+        k.zk_gated_act(ptr(up(rt, gu, dtype)), out.ptr, T, I, act, rt.stream)
+        assert np.abs(rt.download_f32(out) - want).max() <= tol * max(1, np.abs(want).max())
+    z = (rng.normal(size=1001) * 40).astype(np.float32)
+    Z = rt.upload(z)
+    k.zk_softcap(Z.ptr, 1001, 30.0, rt.stream)
+    assert np.abs(rt.download(Z) - 30 * np.tanh(z.astype(np.float64) / 30)).max() < 1e-5
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd,rot,bs,vt", [(4, 2, 16, 16, 4, 0), (6, 1, 32, 32, 8, 1), (8, 4, 256, 256, 16, 1),
+                                                (3, 3, 64, 32, 16, 0), (2, 2, 48, 0, 4, 1)])
+def test_rope_and_cache_write(rt, dtype, nh, nkv, hd, rot, bs, vt):
+    k = rt.kernels(dtype)
+    rng = np.random.default_rng(hd)
+    T, pages = 7, 9
+    qkv = rng.normal(size=(T, (nh + 2 * nkv) * hd)).astype(np.float32)
+    if dtype == "bfloat16":
+        qkv = bf16(qkv)
+    pos = np.array([0, 1, 5, 1000, 8191, 17, 3], np.int32)
+    slots = rng.permutation(pages * bs)[:T].astype(np.int32)
+    slots[2] = -1                                            # nothing stored for this token
+    theta = 10000.0
+    inv = (1.0 / theta ** (2.0 * np.arange(rot // 2) / max(rot, 1))).astype(np.float32)
+    Q = up(rt, qkv, dtype)
+    KC = rt.zeros((pages, nkv, bs, hd), dtype)
+    VC = rt.zeros((pages, nkv, hd, bs) if vt else (pages, nkv, bs, hd), dtype)
+    k.zk_rope_cache_write(Q.ptr, ptr(rt.upload(pos)), ptr(rt.upload(slots)), ptr(rt.upload(inv)) if rot else None, rot,
+                          KC.ptr, VC.ptr, T, nh, nkv, hd, bs, vt, rt.stream)
+
+    def rotate(x):                                           # x [T, heads, hd]
+        x = x.astype(np.float64)
+        if not rot:
+            return x
+        ang = pos[:, None].astype(np.float64) * inv.astype(np.float64)[None, :]
+        c, s = np.cos(ang)[:, None, :], np.sin(ang)[:, None, :]
+        a, b = x[..., :rot // 2], x[..., rot // 2:rot]
+        return np.concatenate([a * c - b * s, b * c + a * s, x[..., rot:]], axis=-1)
+
+    q = qkv[:, :nh * hd].reshape(T, nh, hd)
+    kk = qkv[:, nh * hd:(nh + nkv) * hd].reshape(T, nkv, hd)
+    vv = qkv[:, (nh + nkv) * hd:].reshape(T, nkv, hd)
+    tol = 2e-3 if dtype == "float32" else 0.03               # float angles at position 8191
+    got = rt.download_f32(Q)
+    assert np.abs(got[:, :nh * hd].reshape(T, nh, hd) - rotate(q)).max() < tol
+    assert np.array_equal(got[:, nh * hd:], qkv[:, nh * hd:])            # k and v rows are left as they were
+    kc, vc = rt.download_f32(KC), rt.download_f32(VC)
+    want_k, want_v = np.zeros_like(kc), np.zeros_like(vc)
+    rk = rotate(kk)
+    for t in range(T):
+        if slots[t] < 0:
+            continue
+        p, o = divmod(int(slots[t]), bs)
+        want_k[p, :, o, :] = rk[t]
+        if vt:
+            want_v[p, :, :, o] = vv[t]
+        else:
+            want_v[p, :, o, :] = vv[t]
+    assert np.abs(kc - want_k).max() < tol and np.array_equal(vc, want_v)
+
+
+def test_convert_and_fill(rt):
+    rng = np.random.default_rng(0)
+    x = rng.normal(size=1003).astype(np.float32)
+    from zse_amd.weights.safetensors import f32_to_bf16_bits
+    kb, kf = rt.kernels("bfloat16"), rt.kernels("float32")
+    out = rt.empty((1003,), "bfloat16")
+    kb.zk_convert(ptr(rt.upload(x)), 0, out.ptr, 1, 1003, rt.stream)
+    assert np.array_equal(rt.download(out), f32_to_bf16_bits(x))         # round to nearest even, as on the host
+    half = x.astype(np.float16)
+    out32 = rt.empty((1003,), "float32")
+    kf.zk_convert(ptr(rt.upload(half.view(np.uint16), "bfloat16")), 2, out32.ptr, 0, 1003, rt.stream)
+    assert np.array_equal(rt.download(out32), half.astype(np.float32))
+    kf.zk_convert(ptr(rt.upload(f32_to_bf16_bits(x), "bfloat16")), 1, out32.ptr, 1, 1003, rt.stream)
+    assert np.array_equal(rt.download(out32), bf16(x))
+    big = rt.empty((200001,), "float32")
+    kf.zk_fill_normal(big.ptr, 0, 200001, 5, 9, 0.5, 0.02, rt.stream)
+    a = rt.download(big)
+    assert abs(a.mean() - 0.5) < 3e-4 and abs(a.std() - 0.02) < 3e-4
+    kf.zk_fill_normal(out32.ptr, 0, 1003, 5, 9, 0.5, 0.02, rt.stream)
+    assert np.array_equal(rt.download(out32), a[:1003])                   # a function of (seed, stream, index)
+    kf.zk_fill_normal(out32.ptr, 0, 1003, 6, 9, 0.5, 0.02, rt.stream)
+    assert not np.array_equal(rt.download(out32), a[:1003])
+    kf.zk_zero(big.ptr, 200000, rt.stream)
+    z = rt.download(big)
+    assert not z[:50000].any() and z[50000] != 0
+
+
+def test_argmax_and_sampling(rt):
+    from plain import gemma2_plain as P
+    k = rt.kernels("float32")
+    rng = np.random.default_rng(1)
+    rows, V = 5, 256003
+    z = rng.normal(size=(rows, V)).astype(np.float32) * 3
+    z[1, 777] = z[1, 200000] = 50.0                          # a tie: the lower index wins
+    z[2, V - 1] = 60.0
+    z[3, 5] = np.nan
+    Z = rt.upload(z)
+    ids = rt.empty((rows,), "int32")
+    scratch = rt.empty((rows * 128,), "float32")
+    k.zk_argmax(Z.ptr, ids.ptr, rows, V, scratch.ptr, rt.stream)
+    got = rt.download(ids)
+    want = [int(np.nanargmax(r)) for r in z]
+    want[1] = 777
+    assert list(got) == want
+    # (ref) the sampler vectors of tests/test_orchestrator.py:175-190
+    small = np.array([[0.1, 0.5, 0.3, 0.9, 0.2], [-1.0, -0.5, -2.0, -3.0, -9.0]], np.float32)
+    k.zk_argmax(ptr(rt.upload(small)), ids.ptr, 2, 5, scratch.ptr, rt.stream)
+    assert list(rt.download(ids)[:2]) == [3, 1]
+    # temperature sampling: the plain sampler's draw for the same uniform number
+    z = rng.normal(size=(rows, 1000)).astype(np.float32) * 2
+    temps = np.array([0.8, 1.0, 0.3, 2.0, 1.0], np.float32)
+    us = np.array([0.0, 0.999999, 0.5, 0.25, 0.75])
+    k.zk_sample(ptr(rt.upload(z)), ptr(rt.upload(temps)), ptr(rt.upload(us)), None, ids.ptr, rows, 1000, rt.stream)
+    assert list(rt.download(ids)) == [P.sample(z[i], us[i], temperature=float(temps[i])) for i in range(rows)]
+    # the frequencies follow softmax(z / T)
+    z1 = np.array([[2.0, 1.0, 0.0, -1.0]], np.float32).repeat(4000, 0)
+    from zse_amd.sampling import uniform
+    u = np.array([uniform(3, i) for i in range(4000)])
+    out = rt.empty((4000,), "int32")
+    k.zk_sample(ptr(rt.upload(z1)), ptr(rt.upload(np.full(4000, 0.7, np.float32))), ptr(rt.upload(u)), None, out.ptr,
+                4000, 4, rt.stream)
+    freq = np.bincount(rt.download(out), minlength=4) / 4000.0
+    assert np.abs(freq - P.softmax(z1[0] / 0.7)).max() < 0.03

@@ -45,13 +45,13 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 // ------------------------------------------------------------------ skinny
 // GATED: the block also streams the strip of "up" rows I + n and stores act(g)*u.
-template <int MT, bool GATED>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const __bf16* __restrict__ A, int lda,
+template <int MT, bool GATED, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __restrict__ A, int lda,
                                                           const __bf16* __restrict__ W,
                                                           void* __restrict__ C, int ldc, int c_is_f32,
                                                           int M, int N, int K, int epi, float cap) {
   constexpr int NS = GATED ? 2 : 1;
-  __shared__ f32x4 red[3][NS][MT][64];
+  __shared__ f32x4 red[NW - 1][NS][MT][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, kq = lane >> 4;
   const int n0 = blockIdx.x * 16;
@@ -73,14 +73,17 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const __bf16* __restri
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) acc[s][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  constexpr int STEPS = (MT * NS >= 4) ? 4 : 8;   // 32-wide k steps a wave loads before it multiplies
-  constexpr int KB = STEPS * 32;
-  for (int k0 = wave * KB; k0 < K; k0 += 4 * KB) {
+  // the K range is cut into NW equal runs of 32-wide steps, one run a wave
+  constexpr int STEPS = (MT * NS >= 4) ? 4 : 8;   // steps a wave loads before it multiplies
+  const int total_steps = (K + 31) / 32;
+  const int per_wave = (total_steps + NW - 1) / NW;
+  const int s_begin = wave * per_wave, s_end = min(total_steps, s_begin + per_wave);
+  for (int s0 = s_begin; s0 < s_end; s0 += STEPS) {
     bf16x8 wf[NS][STEPS], af[MT][STEPS];
 #pragma unroll
     for (int s = 0; s < STEPS; s++) {
-      const int k = k0 + s * 32;
-      const bool in = k + kq * 8 < K;
+      const int k = (s0 + s) * 32;
+      const bool in = (s0 + s < s_end) && (k + kq * 8 < K);
 #pragma unroll
       for (int g = 0; g < NS; g++) wf[g][s] = in ? *(const bf16x8*)(wp[g] + k) : zero8();
 #pragma unroll
@@ -108,7 +111,11 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const __bf16* __restri
     const int m = mt * 16 + r;
     f32x4 v[NS];
 #pragma unroll
-    for (int g = 0; g < NS; g++) v[g] = acc[g][mt] + red[0][g][mt][lane] + red[1][g][mt][lane] + red[2][g][mt][lane];
+    for (int g = 0; g < NS; g++) {
+      v[g] = acc[g][mt];
+#pragma unroll
+      for (int w = 0; w < NW - 1; w++) v[g] += red[w][g][mt][lane];
+    }
     if (m >= M) continue;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -251,13 +258,15 @@ static int launch_skinny(const void* A, int lda, const void* W, void* C, int ldc
                          int N, int K, int epi, float cap, hipStream_t s) {
   const int mt = (M + 15) / 16;
   dim3 grid((N + 15) / 16);
-#define ZK_SKINNY(MT_)                                                                          \
-  gemm_skinny_kernel<MT_, GATED><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, \
-                                                      ldc, c_is_f32, M, N, K, epi, cap)
-  if (mt == 1) ZK_SKINNY(1);
-  else if (mt == 2) ZK_SKINNY(2);
-  else if (mt == 3) ZK_SKINNY(3);
-  else ZK_SKINNY(4);
+  // few strips: eight waves a strip keep enough loads in flight
+  const bool wide = grid.x < 512 && K >= 2048 && mt <= 2;
+#define ZK_SKINNY(MT_, NW_)                                                                           \
+  gemm_skinny_kernel<MT_, GATED, NW_><<<grid, NW_ * 64, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, \
+                                                                C, ldc, c_is_f32, M, N, K, epi, cap)
+  if (mt == 1) { if (wide) ZK_SKINNY(1, 8); else ZK_SKINNY(1, 4); }
+  else if (mt == 2) { if (wide) ZK_SKINNY(2, 8); else ZK_SKINNY(2, 4); }
+  else if (mt == 3) ZK_SKINNY(3, 4);
+  else ZK_SKINNY(4, 4);
 #undef ZK_SKINNY
   return zk_launch_status("zk_gemm_bf16 (skinny)");
 }
