@@ -69,6 +69,8 @@ def main():
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
+                    help="profiling aid: run one of the two workloads (the JSON line then lacks the other)")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not measured")
@@ -104,7 +106,7 @@ def main():
     # ---- prefill: one prompt of 2,048 tokens in one step
     T = a.prefill_tokens
     times = []
-    for i in range(4):
+    for i in range(4 if a.only != "decode" else 0):
         toks = rng.integers(0, V, T).tolist()
         rt.sync()
         t1 = time.perf_counter()
@@ -112,11 +114,16 @@ def main():
         rt.sync()
         times.append(time.perf_counter() - t1)
         runner.finish(f"p{i}")
-    pre_s = float(np.median(times[1:]))
-    pf = prefill_flops(cfg, T)
-    prefill = {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
-               "frac": round(pf / pre_s / PEAK_FLOPS["bf16"], 4)}
-    print(f"[bench] prefill {T} tokens: {pre_s * 1e3:.2f} ms", file=sys.stderr, flush=True)
+    prefill = None
+    if times:
+        pre_s = float(np.median(times[1:]))
+        pf = prefill_flops(cfg, T)
+        prefill = {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
+                   "frac": round(pf / pre_s / PEAK_FLOPS["bf16"], 4)}
+        print(f"[bench] prefill {T} tokens: {pre_s * 1e3:.2f} ms", file=sys.stderr, flush=True)
+    if a.only == "prefill":
+        print(json.dumps({"prefill": prefill}), flush=True)
+        return
 
     # ---- decode at each batch size, ending at the full context
     def decode(B, steps, warmup):
