@@ -93,7 +93,7 @@ def main():
     page = 16
     runner = StepRunner(model, rt, "bfloat16", page_size=page,
                         num_pages=max_b * (-(-a.context // page) + 1) + 8, max_seqs=max_b,
-                        max_batch_tokens=max(a.prefill_tokens, max_b), max_model_len=a.context + page,
+                        max_batch_tokens=max(a.prefill_tokens, max_b), max_model_len=a.context,
                         use_graphs=not a.no_graphs)
     sampler = DeviceSampler(rt, runner.k, max_b)
     greedy = SamplingParams(temperature=0.0)

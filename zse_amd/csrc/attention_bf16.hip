@@ -20,9 +20,12 @@
 // the same permutation.  V is therefore cached transposed, [page][kv head][hd][bs],
 // so that four consecutive keys of a channel are one 8-byte load.
 //
-// Decoded tokens use the split variant: the keys are cut into chunks of 128
-// aligned to absolute positions, one wave per chunk writes (max, sum, O) and a
-// second kernel joins the chunks in order; the cut does not depend on the batch.
+// Decoded tokens use a split variant: the keys are cut into chunks of 64 aligned
+// to absolute positions, one wave per chunk writes (max, sum, O) and a second
+// kernel joins the chunks in order; the cut does not depend on the batch.  With
+// at most 16 heads a KV head the chunks run on 16x16x32 MFMAs (attn_decode_kernel):
+// a single query token fills only g of a tile's columns, and the narrower tile
+// halves both the accumulator registers and the wasted work, so two waves fit a SIMD.
 #include "common.h"
 
 #if ZSE_ACT_BF16
@@ -32,7 +35,7 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-#define ATT_CHUNK 128
+#define ATT_CHUNK 64
 
 struct AttnParams {
   const __bf16* q;
@@ -219,6 +222,163 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
   }
 }
 
+// One wave per (request, KV head, chunk of 64 keys) for requests that bring one token.
+// Columns of every tile are the g query heads of the KV head (col = lane % 16), rows are
+// keys (first product) or channels (second product).
+template <int HD32>
+__global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
+  constexpr int KS = HD32;       // 32-wide steps over head_dim
+  constexpr int DT = HD32 * 2;   // 16-channel output tiles
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, kq = lane >> 4;
+  const int r = p.r_begin + blockIdx.z;
+  const int kvh = blockIdx.y;
+  const int chunk = blockIdx.x * 4 + wave;
+  const int n = p.q_start[r + 1] - p.q_start[r];
+  if (n <= 0) return;
+  const int pos = p.ctx_len[r] - 1;
+  const int row_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int key_lo = max(row_lo, chunk * ATT_CHUNK);
+  const int key_hi = min(pos, chunk * ATT_CHUNK + ATT_CHUNK - 1);
+  const bool active = key_lo <= key_hi;          // a wave without keys still meets the others at the barrier
+  const int g = p.nh / p.nkv;
+  const bool col_ok = col < g;
+  const int head = kvh * g + (col_ok ? col : 0);
+  const int trow = p.q_start[r];
+  const int* table = p.block_table + (size_t)r * p.max_blocks;
+  const int hd = p.hd, bs = p.bs, nkv = p.nkv;
+
+  // the query operand waits in LDS (one 16-byte piece per lane and step), not in registers
+  __shared__ bf16x8 sq[4][KS][64];
+  {
+    const __bf16* qr = p.q + (size_t)trow * p.q_stride + (size_t)head * hd + kq * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      bf16x8 t;
+      if (col_ok) t = *(const bf16x8*)(qr + ks * 32);
+      else
+#pragma unroll
+        for (int e = 0; e < 8; e++) t[e] = (__bf16)0.f;
+      sq[wave][ks][lane] = t;
+    }
+  }
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+
+  for (int key0 = (key_lo / 32) * 32; active && key0 <= key_hi; key0 += 32) {
+    bf16x8 kf[2][KS];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      const int kk = min(key0 + 16 * t + col, key_hi);
+      const int page = max(table[kk / bs], 0);
+      const __bf16* kr = p.kcache + (((size_t)page * nkv + kvh) * bs + (kk % bs)) * hd + kq * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) kf[t][ks] = *(const bf16x8*)(kr + ks * 32);
+    }
+    bf16x8 vf[DT];
+    {
+      const int ka = min(key0 + 4 * kq, key_hi & ~3), kb = min(key0 + 16 + 4 * kq, key_hi & ~3);
+      const int pa = max(table[ka / bs], 0), pb = max(table[kb / bs], 0);
+      const __bf16* va_base = p.vcache + ((size_t)pa * nkv + kvh) * hd * bs + (ka % bs);
+      const __bf16* vb_base = p.vcache + ((size_t)pb * nkv + kvh) * hd * bs + (kb % bs);
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++) {
+        const int d = dt * 16 + col;
+        const bf16x4 va = *(const bf16x4*)(va_base + (size_t)d * bs);
+        const bf16x4 vb = *(const bf16x4*)(vb_base + (size_t)d * bs);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          vf[dt][e] = va[e];
+          vf[dt][4 + e] = vb[e];
+        }
+      }
+    }
+    f32x4 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][ks], sq[wave][ks][lane], s[t], 0, 0, 0);
+    }
+    float mt = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int key = key0 + 16 * t + 4 * kq + i;
+        float v = s[t][i] * p.scale;
+        if (p.softcap > 0.f) v = p.softcap * fast_tanh(v / p.softcap);
+        v = (col_ok && key >= key_lo && key <= key_hi) ? v : -INFINITY;
+        s[t][i] = v;
+        mt = fmaxf(mt, v);
+      }
+    mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m_run, mt);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = __expf(m_run - m_use);
+    float rs = 0.f;
+    bf16x8 pb8;
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const float pe = __expf(s[t][i] - m_use);
+        rs += pe;
+        pb8[4 * t + i] = (__bf16)pe;
+      }
+    rs += __shfl_xor(rs, 16, 64);
+    rs += __shfl_xor(rs, 32, 64);
+    l_run = l_run * corr + rs;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+      o[dt] *= corr;
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb8, o[dt], 0, 0, 0);
+    }
+  }
+  // the block's four chunks are joined here, in chunk order: one partial result per 256 keys
+  extern __shared__ float dyn[];
+  float* sm_ml = dyn;                 // [4][16][2]
+  float* sm_o = dyn + 4 * 16 * 2;     // [4][g][hd]
+  if (col_ok) {
+    if (kq == 0) {
+      sm_ml[(wave * 16 + col) * 2] = m_run;
+      sm_ml[(wave * 16 + col) * 2 + 1] = l_run;
+    }
+    float* so = sm_o + ((size_t)wave * g + col) * hd;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) *(f32x4*)(so + dt * 16 + 4 * kq) = o[dt];
+  }
+  __syncthreads();
+  const int first_chunk = blockIdx.x * 4;
+  if (first_chunk * ATT_CHUNK > pos || first_chunk * ATT_CHUNK + 4 * ATT_CHUNK - 1 < row_lo) return;
+  for (int idx = threadIdx.x; idx < g * hd; idx += 256) {
+    const int c = idx / hd, d = idx - c * hd;
+    float mw[4], m = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      mw[w] = sm_ml[(w * 16 + c) * 2];
+      m = fmaxf(m, mw[w]);
+    }
+    float acc = 0.f, l = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      const float e = mw[w] == -INFINITY ? 0.f : __expf(mw[w] - m);
+      acc += e * sm_o[((size_t)w * g + c) * hd + d];
+      l += e * sm_ml[(w * 16 + c) * 2 + 1];
+    }
+    const size_t slot = ((size_t)(r - p.r_begin) * p.nh + kvh * g + c) * p.nchunks + blockIdx.x;
+    p.part_o[slot * hd + d] = acc;
+    if (d == 0) {
+      p.part_ml[slot * 2] = m;
+      p.part_ml[slot * 2 + 1] = l;
+    }
+  }
+}
+
 // Joins the chunks of a decoded token's attention, in chunk order: a block per
 // (request, head), a thread per channel; the chunks' weights exp(m_c - m) are computed once.
 #define ATT_MAX_CHUNKS 1024
@@ -227,7 +387,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
                                                            const int* __restrict__ q_start,
                                                            const int* __restrict__ ctx_len,
                                                            __bf16* __restrict__ out, int nh, int hd,
-                                                           int window, int r_begin, int nchunks) {
+                                                           int window, int r_begin, int nchunks, int span) {
   __shared__ float wgt[ATT_MAX_CHUNKS];
   __shared__ float red[17];
   const int rr = blockIdx.x, head = blockIdx.y;
@@ -236,7 +396,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
   if (n <= 0) return;
   const int pos = ctx_len[r] - 1;
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int c0 = lo / ATT_CHUNK, c1 = pos / ATT_CHUNK;
+  const int c0 = lo / span, c1 = pos / span;
   const size_t base = ((size_t)rr * nh + head) * nchunks;
   float m = -INFINITY;
   for (int c = c0 + threadIdx.x; c <= c1; c += 256) m = fmaxf(m, part_ml[(base + c) * 2]);
@@ -254,9 +414,20 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
   l = block_sum(l, red);
   const float inv = 1.f / l;
   __bf16* orow = out + ((size_t)q_start[r] * nh + head) * hd;
+  const int np = c1 - c0 + 1;
   for (int d = threadIdx.x; d < hd; d += 256) {
+    const float* po = part_o + (base + c0) * hd + d;
     float acc = 0.f;
-    for (int c = c0; c <= c1; c++) acc += part_o[(base + c) * hd + d] * wgt[c - c0];
+    int c = 0;
+    for (; c + 4 <= np; c += 4) {       // four loads in flight, summed in part order
+      const float v0 = po[(size_t)c * hd], v1 = po[(size_t)(c + 1) * hd];
+      const float v2 = po[(size_t)(c + 2) * hd], v3 = po[(size_t)(c + 3) * hd];
+      acc += v0 * wgt[c];
+      acc += v1 * wgt[c + 1];
+      acc += v2 * wgt[c + 2];
+      acc += v3 * wgt[c + 3];
+    }
+    for (; c < np; c++) acc += po[(size_t)c * hd] * wgt[c];
     orow[d] = (__bf16)(acc * inv);
   }
 }
@@ -286,7 +457,7 @@ int zk_attention_bf16_supports(int nh, int nkv, int hd, int bs) {
 
 // Bytes of workspace the split variant needs for ``n_decode`` single-token requests.
 size_t zk_attention_bf16_workspace(int n_decode, int nh, int hd, int max_ctx) {
-  const size_t nchunks = ((size_t)max_ctx + ATT_CHUNK - 1) / ATT_CHUNK;
+  const size_t nchunks = ((size_t)max_ctx + ATT_CHUNK - 1) / ATT_CHUNK;      // an upper bound for both variants
   return (size_t)n_decode * nh * nchunks * (hd + 2) * sizeof(float);
 }
 
@@ -331,12 +502,29 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
     p.part_o = (float*)workspace;
     p.part_ml = (float*)workspace + (size_t)n_dec * nh * nchunks * hd;
     dim3 grid((nchunks + 3) / 4, nkv, n_dec);
-    int rc = launch_attn<true>(p, grid, s);
+    int rc = 0;
+    int span = ATT_CHUNK;        // keys one partial result covers
+    if (g <= 16 && hd % 32 == 0) {
+      // the block joins its four chunks: one partial result per 4 * ATT_CHUNK keys
+      span = 4 * ATT_CHUNK;
+      p.nchunks = grid.x;
+      p.part_ml = (float*)workspace + (size_t)n_dec * nh * p.nchunks * hd;
+      const size_t lds = (4 * 16 * 2 + (size_t)4 * g * hd) * sizeof(float);
+      switch (hd / 32) {
+        case 1: attn_decode_kernel<1><<<grid, 256, lds, s>>>(p); break;
+        case 2: attn_decode_kernel<2><<<grid, 256, lds, s>>>(p); break;
+        case 4: attn_decode_kernel<4><<<grid, 256, lds, s>>>(p); break;
+        default: attn_decode_kernel<8><<<grid, 256, lds, s>>>(p); break;
+      }
+      rc = zk_launch_status("zk_attention_bf16 (decode)");
+    } else {
+      rc = launch_attn<true>(p, grid, s);
+    }
     if (rc) return rc;
     ZK_REQUIRE(nchunks <= ATT_MAX_CHUNKS, "zk_attention_bf16: context too long for the split variant");
     dim3 cgrid(n_dec, nh);
     attn_combine_kernel<<<cgrid, 256, 0, s>>>(p.part_o, p.part_ml, q_start, ctx_len, (__bf16*)out, nh, hd,
-                                             window, r_prefill, nchunks);
+                                              window, r_prefill, p.nchunks, span);
     return zk_launch_status("zk_attention_bf16 (combine)");
   }
   return 0;
