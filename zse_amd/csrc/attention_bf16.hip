@@ -50,7 +50,12 @@ struct AttnParams {
   float* part_o;          // split: [slot][hd]
   float* part_ml;         // split: [slot][2]
   int nh, nkv, hd, bs;
+  int bs_shift;           // page size is 1 << bs_shift in the tuned kernels
   float scale, softcap;
+  // scores in the log2 domain: with a cap c,  s2 = c2 * tanh(k2 * dot / 2)  computed as
+  // c2 * (1 - 2 / (exp2(k2 * dot) + 1)),  k2 = 2 * scale / c * log2(e),  c2 = c * log2(e);
+  // without a cap  s2 = k1 * dot,  k1 = scale * log2(e).  Probabilities are exp2(s2 - m2).
+  float k1, k2, c2;
   int window;
   int tpw;                // tokens a wave owns
   int r_begin;            // first request of this launch
@@ -63,6 +68,14 @@ __device__ __forceinline__ float fast_tanh(float x) {
   return 1.f - 2.f / (e + 1.f);
 }
 
+__device__ __forceinline__ float score_log2(const AttnParams& p, float dot) {
+  if (p.softcap > 0.f) {
+    const float e = __builtin_amdgcn_exp2f(p.k2 * dot);
+    return p.c2 * (1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f));
+  }
+  return p.k1 * dot;
+}
+
 template <int HD16, bool SPLIT>
 __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
   constexpr int DT = (HD16 + 1) / 2;
@@ -73,7 +86,9 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
   const int qs = p.q_start[r], n = p.q_start[r + 1] - qs;
   if (n <= 0) return;
   const int start = p.ctx_len[r] - n;
-  const int gi = SPLIT ? 0 : blockIdx.x * 4 + wave;
+  // portions: a block owns one group of rows and its four waves take every fourth tile of
+  // keys (their results are joined at the end); decoded tokens: a wave owns one chunk of keys
+  const int gi = SPLIT ? 0 : blockIdx.x;
   const int chunk = SPLIT ? blockIdx.x * 4 + wave : 0;
   const int t0 = gi * p.tpw;
   if (t0 >= n) return;
@@ -91,10 +106,10 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
     key_lo = max(key_lo, chunk * ATT_CHUNK);
     key_hi = min(key_hi, chunk * ATT_CHUNK + ATT_CHUNK - 1);
   }
-  if (key_lo > key_hi) return;
+  if (SPLIT && key_lo > key_hi) return;
   const int row_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
   const int* table = p.block_table + (size_t)r * p.max_blocks;
-  const int hd = p.hd, bs = p.bs, nkv = p.nkv;
+  const int hd = p.hd, bsh = p.bs_shift, bmask = p.bs - 1, nkv = p.nkv;
 
   bf16x8 qf[HD16];
   {
@@ -114,15 +129,15 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
     for (int e = 0; e < 16; e++) o[dt][e] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  for (int key0 = (key_lo / 32) * 32; key0 <= key_hi; key0 += 32) {
+  for (int key0 = (key_lo / 32) * 32 + (SPLIT ? 0 : wave * 32); key0 <= key_hi; key0 += SPLIT ? 32 : 128) {
     // ---- S^T = K Q^T
     f32x16 s;
 #pragma unroll
     for (int e = 0; e < 16; e++) s[e] = 0.f;
     {
       const int kk = min(key0 + lr, key_hi);
-      const int page = max(table[kk / bs], 0);
-      const __bf16* kr = p.kcache + (((size_t)page * nkv + kvh) * bs + (kk % bs)) * hd + lk * 8;
+      const int page = max(table[kk >> bsh], 0);
+      const __bf16* kr = p.kcache + ((((size_t)page * nkv + kvh) << bsh) + (kk & bmask)) * hd + lk * 8;
       bf16x8 kf[HD16];
 #pragma unroll
       for (int ks = 0; ks < HD16; ks++) kf[ks] = *(const bf16x8*)(kr + ks * 16);
@@ -134,12 +149,12 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
 #pragma unroll
     for (int h = 0; h < 2; h++) {
       const int ka = min(key0 + h * 16 + 4 * lk, key_hi & ~3), kb = min(key0 + h * 16 + 8 + 4 * lk, key_hi & ~3);
-      const int pa = max(table[ka / bs], 0), pb = max(table[kb / bs], 0);
+      const int pa = max(table[ka >> bsh], 0), pb = max(table[kb >> bsh], 0);
 #pragma unroll
       for (int dt = 0; dt < DT; dt++) {
         const int d = min(dt * 32 + lr, hd - 1);
-        const bf16x4 va = *(const bf16x4*)(p.vcache + (((size_t)pa * nkv + kvh) * hd + d) * bs + (ka % bs));
-        const bf16x4 vb = *(const bf16x4*)(p.vcache + (((size_t)pb * nkv + kvh) * hd + d) * bs + (kb % bs));
+        const bf16x4 va = *(const bf16x4*)(p.vcache + (((((size_t)pa * nkv + kvh) * hd + d)) << bsh) + (ka & bmask));
+        const bf16x4 vb = *(const bf16x4*)(p.vcache + (((((size_t)pb * nkv + kvh) * hd + d)) << bsh) + (kb & bmask));
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           vf[dt][h][e] = va[e];
@@ -154,21 +169,21 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int key = key0 + 8 * j + 4 * lk + i;
-        float v = s[4 * j + i] * p.scale;
-        if (p.softcap > 0.f) v = p.softcap * fast_tanh(v / p.softcap);
+        float v = score_log2(p, s[4 * j + i]);
         const bool ok = row_ok && key >= row_lo && key <= pos && key >= key_lo && key <= key_hi;
         v = ok ? v : -INFINITY;
         s[4 * j + i] = v;
         mt = fmaxf(mt, v);
       }
     mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-    const float m_new = fmaxf(m_run, mt);
+    const float m_new = mt > m_run + 8.f ? mt : m_run;      // the reference follows the maximum lazily
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float corr = __expf(m_run - m_use);
+    const bool moved = m_new > m_run;
+    const float corr = moved ? __builtin_amdgcn_exp2f(m_run - m_use) : 1.f;
     float rs = 0.f;
 #pragma unroll
     for (int e = 0; e < 16; e++) {
-      const float pe = __expf(s[e] - m_use);
+      const float pe = __builtin_amdgcn_exp2f(s[e] - m_use);
       s[e] = pe;
       rs += pe;
     }
@@ -181,16 +196,20 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
 #pragma unroll
       for (int e = 0; e < 8; e++) pb[h][e] = (__bf16)s[8 * h + e];
     // ---- O^T = corr * O^T + V^T P^T
+    if (__any(moved)) {
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) o[dt][e] *= corr;
+    }
 #pragma unroll
     for (int dt = 0; dt < DT; dt++) {
-#pragma unroll
-      for (int e = 0; e < 16; e++) o[dt][e] *= corr;
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][0], pb[0], o[dt], 0, 0, 0);
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][1], pb[1], o[dt], 0, 0, 0);
     }
   }
-  if (!row_ok) return;
   if (SPLIT) {
+    if (!row_ok) return;
     const size_t slot = ((size_t)(r - p.r_begin) * p.nh + head) * p.nchunks + chunk;
     if (lk == 0) {
       p.part_ml[slot * 2] = m_run;
@@ -205,7 +224,59 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
         if (d < hd) *(f32x4*)(po + d) = f32x4{o[dt][4 * j], o[dt][4 * j + 1], o[dt][4 * j + 2], o[dt][4 * j + 3]};
       }
   } else {
-    const float inv = 1.f / l_run;
+    // join the four waves' partial results: common maximum and sum per row, then the
+    // accumulators meet in LDS (waves 2, 3 -> 0, 1; then 1 -> 0)
+    extern __shared__ float dyn[];
+    float* sm_ml = dyn;                          // [4][32][2]
+    float* sm_o = dyn + 4 * 32 * 2;              // [2][DT * 16][64]
+    if (lk == 0) {
+      sm_ml[(wave * 32 + lr) * 2] = m_run;
+      sm_ml[(wave * 32 + lr) * 2 + 1] = l_run;
+    }
+    __syncthreads();
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; w++) m_all = fmaxf(m_all, sm_ml[(w * 32 + lr) * 2]);
+    float l_all = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      const float mw = sm_ml[(w * 32 + lr) * 2];
+      l_all += mw == -INFINITY ? 0.f : sm_ml[(w * 32 + lr) * 2 + 1] * __builtin_amdgcn_exp2f(mw - m_all);
+    }
+    const float f = m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - m_all);
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) o[dt][e] *= f;
+    if (wave >= 2) {
+      float* dst = sm_o + (size_t)(wave - 2) * DT * 16 * 64;
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) dst[(dt * 16 + e) * 64 + lane] = o[dt][e];
+    }
+    __syncthreads();
+    if (wave < 2) {
+      const float* src = sm_o + (size_t)wave * DT * 16 * 64;
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) o[dt][e] += src[(dt * 16 + e) * 64 + lane];
+    }
+    __syncthreads();
+    if (wave == 1) {
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) sm_o[(dt * 16 + e) * 64 + lane] = o[dt][e];
+    }
+    __syncthreads();
+    if (wave != 0 || !row_ok) return;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) o[dt][e] += sm_o[(dt * 16 + e) * 64 + lane];
+    const float inv = 1.f / l_all;
     __bf16* orow = p.out + ((size_t)trow * p.nh + head) * hd;
 #pragma unroll
     for (int dt = 0; dt < DT; dt++)
@@ -246,7 +317,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const int head = kvh * g + (col_ok ? col : 0);
   const int trow = p.q_start[r];
   const int* table = p.block_table + (size_t)r * p.max_blocks;
-  const int hd = p.hd, bs = p.bs, nkv = p.nkv;
+  const int hd = p.hd, bsh = p.bs_shift, bmask = p.bs - 1, nkv = p.nkv;
 
   // the query operand waits in LDS (one 16-byte piece per lane and step), not in registers
   __shared__ bf16x8 sq[4][KS][64];
@@ -272,22 +343,22 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
     for (int t = 0; t < 2; t++) {
       const int kk = min(key0 + 16 * t + col, key_hi);
-      const int page = max(table[kk / bs], 0);
-      const __bf16* kr = p.kcache + (((size_t)page * nkv + kvh) * bs + (kk % bs)) * hd + kq * 8;
+      const int page = max(table[kk >> bsh], 0);
+      const __bf16* kr = p.kcache + ((((size_t)page * nkv + kvh) << bsh) + (kk & bmask)) * hd + kq * 8;
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) kf[t][ks] = *(const bf16x8*)(kr + ks * 32);
     }
     bf16x8 vf[DT];
     {
       const int ka = min(key0 + 4 * kq, key_hi & ~3), kb = min(key0 + 16 + 4 * kq, key_hi & ~3);
-      const int pa = max(table[ka / bs], 0), pb = max(table[kb / bs], 0);
-      const __bf16* va_base = p.vcache + ((size_t)pa * nkv + kvh) * hd * bs + (ka % bs);
-      const __bf16* vb_base = p.vcache + ((size_t)pb * nkv + kvh) * hd * bs + (kb % bs);
+      const int pa = max(table[ka >> bsh], 0), pb = max(table[kb >> bsh], 0);
+      const __bf16* va_base = p.vcache + ((((size_t)pa * nkv + kvh) * hd) << bsh) + (ka & bmask);
+      const __bf16* vb_base = p.vcache + ((((size_t)pb * nkv + kvh) * hd) << bsh) + (kb & bmask);
 #pragma unroll
       for (int dt = 0; dt < DT; dt++) {
         const int d = dt * 16 + col;
-        const bf16x4 va = *(const bf16x4*)(va_base + (size_t)d * bs);
-        const bf16x4 vb = *(const bf16x4*)(vb_base + (size_t)d * bs);
+        const bf16x4 va = *(const bf16x4*)(va_base + ((size_t)d << bsh));
+        const bf16x4 vb = *(const bf16x4*)(vb_base + ((size_t)d << bsh));
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           vf[dt][e] = va[e];
@@ -308,8 +379,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int key = key0 + 16 * t + 4 * kq + i;
-        float v = s[t][i] * p.scale;
-        if (p.softcap > 0.f) v = p.softcap * fast_tanh(v / p.softcap);
+        float v = score_log2(p, s[t][i]);
         v = (col_ok && key >= key_lo && key <= key_hi) ? v : -INFINITY;
         s[t][i] = v;
         mt = fmaxf(mt, v);
@@ -318,14 +388,14 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
     const float m_new = fmaxf(m_run, mt);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float corr = __expf(m_run - m_use);
+    const float corr = __builtin_amdgcn_exp2f(m_run - m_use);
     float rs = 0.f;
     bf16x8 pb8;
 #pragma unroll
     for (int t = 0; t < 2; t++)
 #pragma unroll
       for (int i = 0; i < 4; i++) {
-        const float pe = __expf(s[t][i] - m_use);
+        const float pe = __builtin_amdgcn_exp2f(s[t][i] - m_use);
         rs += pe;
         pb8[4 * t + i] = (__bf16)pe;
       }
@@ -366,7 +436,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     float acc = 0.f, l = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; w++) {
-      const float e = mw[w] == -INFINITY ? 0.f : __expf(mw[w] - m);
+      const float e = mw[w] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw[w] - m);
       acc += e * sm_o[((size_t)w * g + c) * hd + d];
       l += e * sm_ml[(w * 16 + c) * 2 + 1];
     }
@@ -407,7 +477,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
   __syncthreads();
   float l = 0.f;
   for (int c = c0 + threadIdx.x; c <= c1; c += 256) {
-    const float w = __expf(part_ml[(base + c) * 2] - m);
+    const float w = __builtin_amdgcn_exp2f(part_ml[(base + c) * 2] - m);
     wgt[c - c0] = w;
     l += part_ml[(base + c) * 2 + 1] * w;
   }
@@ -434,12 +504,14 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
 
 template <bool SPLIT>
 static int launch_attn(const AttnParams& p, dim3 grid, hipStream_t s) {
+  // the join of a portion's four waves needs [4][32][2] + [2][ceil(hd/32) * 16][64] floats of LDS
+  const size_t lds = SPLIT ? 0 : (4 * 32 * 2 + (size_t)2 * ((p.hd + 31) / 32) * 16 * 64) * sizeof(float);
   switch (p.hd / 16) {
-    case 1: attn_mfma_kernel<1, SPLIT><<<grid, 256, 0, s>>>(p); break;
-    case 2: attn_mfma_kernel<2, SPLIT><<<grid, 256, 0, s>>>(p); break;
-    case 4: attn_mfma_kernel<4, SPLIT><<<grid, 256, 0, s>>>(p); break;
-    case 8: attn_mfma_kernel<8, SPLIT><<<grid, 256, 0, s>>>(p); break;
-    case 16: attn_mfma_kernel<16, SPLIT><<<grid, 256, 0, s>>>(p); break;
+    case 1: attn_mfma_kernel<1, SPLIT><<<grid, 256, lds, s>>>(p); break;
+    case 2: attn_mfma_kernel<2, SPLIT><<<grid, 256, lds, s>>>(p); break;
+    case 4: attn_mfma_kernel<4, SPLIT><<<grid, 256, lds, s>>>(p); break;
+    case 8: attn_mfma_kernel<8, SPLIT><<<grid, 256, lds, s>>>(p); break;
+    case 16: attn_mfma_kernel<16, SPLIT><<<grid, 256, lds, s>>>(p); break;
     default: return zk_fail("zk_attention_bf16: head_dim must be 16, 32, 64, 128 or 256");
   }
   return zk_launch_status("zk_attention_bf16");
@@ -452,7 +524,7 @@ int zk_attention_bf16_supports(int nh, int nkv, int hd, int bs) {
   if (nkv <= 0 || nh % nkv) return 0;
   const int g = nh / nkv;
   const bool hd_ok = hd == 16 || hd == 32 || hd == 64 || hd == 128 || hd == 256;
-  return hd_ok && g <= 32 && bs % 4 == 0;
+  return hd_ok && g <= 32 && bs >= 4 && (bs & (bs - 1)) == 0;
 }
 
 // Bytes of workspace the split variant needs for ``n_decode`` single-token requests.
@@ -470,7 +542,7 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
                       size_t workspace_bytes, void* stream) {
   ZK_REQUIRE(R >= 0 && r_prefill >= 0 && r_prefill <= R, "zk_attention_bf16: bad request counts");
   ZK_REQUIRE(zk_attention_bf16_supports(nh, nkv, hd, bs), "zk_attention_bf16: sizes not supported "
-             "(head_dim 16/32/64/128/256, at most 32 heads a KV head, page size a multiple of 4)");
+             "(head_dim 16/32/64/128/256, at most 32 heads a KV head, page size a power of two from 4)");
   ZK_REQUIRE(q_stride >= nh * hd && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0),
              "zk_attention_bf16: q rows must be 16-byte aligned");
   ZK_REQUIRE(max_blocks > 0 && nkv <= 65535 && R <= 65535, "zk_attention_bf16: grid too large");
@@ -483,12 +555,18 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
   p.q_start = q_start; p.ctx_len = ctx_len; p.out = (__bf16*)out;
   p.nh = nh; p.nkv = nkv; p.hd = hd; p.bs = bs;
   p.scale = scale; p.softcap = softcap; p.window = window;
+  p.bs_shift = 0;
+  while ((1 << p.bs_shift) < bs) p.bs_shift++;
+  const float log2e = 1.4426950408889634f;
+  p.k1 = scale * log2e;
+  p.k2 = softcap > 0.f ? 2.f * scale / softcap * log2e : 0.f;
+  p.c2 = softcap * log2e;
   const int g = nh / nkv;
   if (r_prefill > 0) {
     ZK_REQUIRE(max_q_len > 0, "zk_attention_bf16: max_q_len must be positive");
     p.tpw = 32 / g; p.r_begin = 0; p.nchunks = 1; p.part_o = nullptr; p.part_ml = nullptr;
     const int groups = (max_q_len + p.tpw - 1) / p.tpw;
-    dim3 grid((groups + 3) / 4, nkv, r_prefill);
+    dim3 grid(groups, nkv, r_prefill);
     int rc = launch_attn<false>(p, grid, s);
     if (rc) return rc;
   }
