@@ -7,8 +7,8 @@
 //    16x16x32 MFMAs straight from global memory: a lane's 16-byte load is exactly
 //    its MFMA operand (row = lane % 16, eight k values at 8 * (lane / 16)), so no
 //    LDS staging is needed.  Partial sums of the four waves meet in LDS.
-//  * tile (M > 64, prefill): 128x128x64 block tiles staged through LDS, four waves
-//    of 64 lanes, each a 64x64 corner built from 32x32x16 MFMAs.
+//  * tile (M > 64, prefill): 256x128x64 or 128x128x64 block tiles staged through LDS, four waves
+//    of 64 lanes, each a 128x64 or 64x64 corner built from 32x32x16 MFMAs.
 // Epilogues: plain store (bf16 or float), soft cap on float output (LM head), and
 // the gated activation act(gate) * up over a [2I, K] weight whose first I rows are
 // the gate (the feed-forward's first product; the [T, 2I] intermediate never
@@ -73,22 +73,25 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) acc[s][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // the K range is cut into NW equal runs of 32-wide steps, one run a wave
-  constexpr int STEPS = (MT * NS >= 4) ? 4 : 8;   // steps a wave loads before it multiplies
+  // the K range is cut into NW equal runs of 32-wide steps, one run a wave.  A wave works in
+  // groups of STEPS steps and keeps the next group's loads in flight while it multiplies the
+  // current one (two register sets, the loop is unrolled by two to name them).
+  constexpr int STEPS = (MT * NS >= 4) ? 4 : 8;
   const int total_steps = (K + 31) / 32;
   const int per_wave = (total_steps + NW - 1) / NW;
   const int s_begin = wave * per_wave, s_end = min(total_steps, s_begin + per_wave);
-  for (int s0 = s_begin; s0 < s_end; s0 += STEPS) {
-    bf16x8 wf[NS][STEPS], af[MT][STEPS];
+  auto fetch = [&](int s0, bf16x8 (&wf)[NS][STEPS], bf16x8 (&af)[MT][STEPS]) {
 #pragma unroll
     for (int s = 0; s < STEPS; s++) {
       const int k = (s0 + s) * 32;
       const bool in = (s0 + s < s_end) && (k + kq * 8 < K);
 #pragma unroll
-      for (int g = 0; g < NS; g++) wf[g][s] = in ? *(const bf16x8*)(wp[g] + k) : zero8();
-#pragma unroll
       for (int mt = 0; mt < MT; mt++) af[mt][s] = (in && av[mt]) ? *(const bf16x8*)(ap[mt] + k) : zero8();
+#pragma unroll
+      for (int g = 0; g < NS; g++) wf[g][s] = in ? *(const bf16x8*)(wp[g] + k) : zero8();
     }
+  };
+  auto multiply = [&](const bf16x8 (&wf)[NS][STEPS], const bf16x8 (&af)[MT][STEPS]) {
 #pragma unroll
     for (int s = 0; s < STEPS; s++)
 #pragma unroll
@@ -96,6 +99,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
           acc[g][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][s], af[mt][s], acc[g][mt], 0, 0, 0);
+  };
+  bf16x8 wf0[NS][STEPS], af0[MT][STEPS], wf1[NS][STEPS], af1[MT][STEPS];
+  if (s_begin < s_end) fetch(s_begin, wf0, af0);
+  for (int s0 = s_begin; s0 < s_end; s0 += 2 * STEPS) {
+    if (s0 + STEPS < s_end) fetch(s0 + STEPS, wf1, af1);
+    multiply(wf0, af0);
+    if (s0 + STEPS >= s_end) break;
+    if (s0 + 2 * STEPS < s_end) fetch(s0 + 2 * STEPS, wf0, af0);
+    multiply(wf1, af1);
   }
   if (wave > 0) {
 #pragma unroll
@@ -131,91 +143,94 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
 }
 
 // ------------------------------------------------------------------ tile
-#define GT_BM 128
+// Block tile (64 * WMT) x 128 x 64, four waves as 2 x 2, a wave owns WMT x 2 MFMA tiles of
+// 32 x 32.  WMT = 4 (256 x 128 blocks, 128 x 64 a wave) needs 6 operand fragments from LDS
+// for 8 MFMAs where WMT = 2 (128 x 128, 64 x 64 a wave) needs 4 for 4: LDS delivers 128
+// bytes a clock, one fragment per MFMA slot, so the larger wave tile is what lets the matrix
+// cores run ahead of LDS.  The smaller block is kept for shapes that would give too few blocks.
 #define GT_BN 128
 #define GT_BK 64
 #define GT_LD (GT_BK + 8)
 
-template <bool GATED>
+template <int WMT, bool GATED>
 __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict__ A, int lda,
                                                         const __bf16* __restrict__ W,
                                                         void* __restrict__ C, int ldc, int c_is_f32,
                                                         int M, int N, int K, int epi, float cap,
                                                         int tiles_m, int tiles_n) {
-  __shared__ __bf16 sA[GT_BM][GT_LD];
+  constexpr int BM = 64 * WMT;
+  constexpr int APT = BM / 32;                 // 16-byte pieces of A a thread moves per k tile
+  __shared__ __bf16 sA[BM][GT_LD];
   __shared__ __bf16 sB[GT_BN][GT_LD];
   // blocks that share a weight tile run on one XCD (ids go round-robin over 8 XCDs)
   int id = blockIdx.x;
   const int total = tiles_m * tiles_n;
   if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
   const int tn = id / tiles_m, tm = id % tiles_m;
-  const int m0 = tm * GT_BM;
+  const int m0 = tm * BM;
   const int ncols = GATED ? GT_BN / 2 : GT_BN;       // output columns of the block
   const int n0 = tn * ncols;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int lr = lane & 31, lk = lane >> 5;
 
-  // each thread moves four 16-byte pieces of A and of B per k tile
-  const __bf16* ga[4];
+  // piece c = tid + 256 i of a tile: row c / 8, eight k values at (c % 8) * 8
+  const int prow = tid >> 3, pcol = (tid & 7) * 8;
+  const __bf16* ga[APT];
   const __bf16* gb[4];
-  int srow[4], scol[4];
+#pragma unroll
+  for (int i = 0; i < APT; i++) ga[i] = A + (size_t)min(m0 + prow + 32 * i, M - 1) * lda + pcol;
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    const int c = tid + i * 256;
-    srow[i] = c >> 3;
-    scol[i] = (c & 7) * 8;
-    const int am = min(m0 + srow[i], M - 1);
-    ga[i] = A + (size_t)am * lda + scol[i];
+    const int row = prow + 32 * i;
     int bn;
-    if (GATED) bn = srow[i] < 64 ? min(n0 + srow[i], N - 1) : N + min(n0 + srow[i] - 64, N - 1);
-    else bn = min(n0 + srow[i], N - 1);
-    gb[i] = W + (size_t)bn * K + scol[i];
+    if (GATED) bn = row < 64 ? min(n0 + row, N - 1) : N + min(n0 + row - 64, N - 1);
+    else bn = min(n0 + row, N - 1);
+    gb[i] = W + (size_t)bn * K + pcol;
   }
-  f32x16 acc[2][2];
+  f32x16 acc[WMT][2];
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+  for (int i = 0; i < WMT; i++)
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-  bf16x8 ra[4], rb[4];
+  bf16x8 ra[APT], rb[4];
+  {
+    const bool in = pcol < K;
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const bool in = scol[i] < K;
-    ra[i] = in ? *(const bf16x8*)(ga[i]) : zero8();
-    rb[i] = in ? *(const bf16x8*)(gb[i]) : zero8();
+    for (int i = 0; i < APT; i++) ra[i] = in ? *(const bf16x8*)(ga[i]) : zero8();
+#pragma unroll
+    for (int i = 0; i < 4; i++) rb[i] = in ? *(const bf16x8*)(gb[i]) : zero8();
   }
   for (int k0 = 0; k0 < K; k0 += GT_BK) {
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      *(bf16x8*)(&sA[srow[i]][scol[i]]) = ra[i];
-      *(bf16x8*)(&sB[srow[i]][scol[i]]) = rb[i];
-    }
+    for (int i = 0; i < APT; i++) *(bf16x8*)(&sA[prow + 32 * i][pcol]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < 4; i++) *(bf16x8*)(&sB[prow + 32 * i][pcol]) = rb[i];
     __syncthreads();
     const int kn = k0 + GT_BK;
     if (kn < K) {
+      const bool in = kn + pcol < K;
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const bool in = kn + scol[i] < K;
-        ra[i] = in ? *(const bf16x8*)(ga[i] + kn) : zero8();
-        rb[i] = in ? *(const bf16x8*)(gb[i] + kn) : zero8();
-      }
+      for (int i = 0; i < APT; i++) ra[i] = in ? *(const bf16x8*)(ga[i] + kn) : zero8();
+#pragma unroll
+      for (int i = 0; i < 4; i++) rb[i] = in ? *(const bf16x8*)(gb[i] + kn) : zero8();
     }
 #pragma unroll
     for (int ks = 0; ks < GT_BK / 16; ks++) {
-      bf16x8 fa[2], fb[2];
+      bf16x8 fa[WMT], fb[2];
 #pragma unroll
-      for (int i = 0; i < 2; i++) fa[i] = *(const bf16x8*)(&sA[wm * 64 + i * 32 + lr][ks * 16 + lk * 8]);
+      for (int i = 0; i < WMT; i++) fa[i] = *(const bf16x8*)(&sA[wm * (32 * WMT) + i * 32 + lr][ks * 16 + lk * 8]);
 #pragma unroll
       for (int j = 0; j < 2; j++) {
         const int brow = GATED ? j * 64 + wn * 32 : wn * 64 + j * 32;
         fb[j] = *(const bf16x8*)(&sB[brow + lr][ks * 16 + lk * 8]);
       }
 #pragma unroll
-      for (int i = 0; i < 2; i++)
+      for (int i = 0; i < WMT; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
@@ -223,12 +238,12 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
   }
   // acc[i][j][4*b + e] is row 8*b + 4*lk + e of the 32x32 tile, column lr
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
+  for (int i = 0; i < WMT; i++) {
 #pragma unroll
     for (int b = 0; b < 4; b++) {
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        const int m = m0 + wm * 64 + i * 32 + 8 * b + 4 * lk + e;
+        const int m = m0 + wm * (32 * WMT) + i * 32 + 8 * b + 4 * lk + e;
         if (m >= M) continue;
         if (GATED) {
           const int n = n0 + wn * 32 + lr;
@@ -252,6 +267,7 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
     }
   }
 }
+
 
 template <bool GATED>
 static int launch_skinny(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M,
@@ -288,17 +304,21 @@ extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int 
     return gated ? launch_skinny<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, s)
                  : launch_skinny<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, s);
   }
-  const int tiles_m = (M + GT_BM - 1) / GT_BM;
   const int ncols = gated ? GT_BN / 2 : GT_BN;
   const int tiles_n = (N + ncols - 1) / ncols;
+  // 128-row blocks (WMT = 2): three of them fit a CU and hide each other's waits.  The
+  // 256-row block (WMT = 4) halves LDS traffic per MFMA but runs one block a CU with its
+  // loads exposed; measured slower (608 vs 741 TFLOP/s at 2048 x 4096 x 2304) until the k loop
+  // is double-buffered, so it is not selected.
+  const int tiles_m = (M + 127) / 128;
   ZK_REQUIRE((long long)tiles_m * tiles_n < 2147483647LL, "zk_gemm_bf16: too many tiles");
   dim3 grid(tiles_m * tiles_n);
   if (gated)
-    gemm_tile_kernel<true><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32,
-                                                M, N, K, epi, cap, tiles_m, tiles_n);
+    gemm_tile_kernel<2, true><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32,
+                                                   M, N, K, epi, cap, tiles_m, tiles_n);
   else
-    gemm_tile_kernel<false><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32,
-                                                 M, N, K, epi, cap, tiles_m, tiles_n);
+    gemm_tile_kernel<2, false><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32,
+                                                    M, N, K, epi, cap, tiles_m, tiles_n);
   return zk_launch_status("zk_gemm_bf16 (tile)");
 }
 
