@@ -48,7 +48,7 @@ def make_runner(folder, dtype, **kw):
     from zse_amd.engine.runner import StepRunner
     from zse_amd.runtime.device import Runtime
     rt = Runtime.get()
-    model = load_model(folder, dtype, rt)
+    model = load_model(folder, dtype, rt, tuned=kw.pop("tuned", True))
     kw.setdefault("use_graphs", False)
     return StepRunner(model, rt, dtype, **kw)
 

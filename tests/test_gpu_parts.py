@@ -16,7 +16,7 @@ class Weights:
     def __init__(self, rt, dtype, arrays):
         self.rt, self.dtype, self.arrays = rt, dtype, arrays
 
-    def matrix(self, names):
+    def matrix(self, names, strip=False):
         from zse_amd.weights.safetensors import f32_to_bf16_bits
         a = np.concatenate([self.arrays[n] for n in names]).astype(np.float32)
         return self.rt.upload(f32_to_bf16_bits(a), "bfloat16") if self.dtype == "bfloat16" else self.rt.upload(a)

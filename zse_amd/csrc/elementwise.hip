@@ -25,14 +25,22 @@ int zk_launch_status(const char* what) {
 
 // ------------------------------------------------------------------ embedding
 
+// strip: the table is in the matrix-core kernels' strip layout (element (n, k) at
+// ((n/16 * (H/32) + k/32) * 64 + (k%32)/8 * 16 + n%16) * 8 + k%8) instead of row-major.
 template <typename W>
 __global__ void embed_kernel(const W* __restrict__ table, const int* __restrict__ tokens,
-                             float* __restrict__ out, float scale, int H, int V) {
+                             float* __restrict__ out, float scale, int H, int V, int strip) {
   const int t = blockIdx.x;
   int tok = tokens[t];
   tok = tok < 0 ? 0 : (tok >= V ? V - 1 : tok);
-  const W* row = table + (size_t)tok * H;
   float* o = out + (size_t)t * H;
+  if (strip) {
+    const size_t base = (size_t)(tok >> 4) * (H / 32) * 512 + (tok & 15) * 8;
+    for (int i = threadIdx.x; i < H; i += blockDim.x)
+      o[i] = to_f32(table[base + (size_t)(i >> 5) * 512 + ((i & 31) >> 3) * 128 + (i & 7)]) * scale;
+    return;
+  }
+  const W* row = table + (size_t)tok * H;
   for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32(row[i]) * scale;
 }
 
@@ -352,10 +360,11 @@ const char* zk_last_error() { return zk_error.c_str(); }
 int zk_act_is_bf16() { return ZSE_ACT_BF16; }
 
 int zk_embed(const void* table, const int* tokens, float* out, float scale, int T, int H, int V,
-             void* stream) {
+             int strip, void* stream) {
   ZK_REQUIRE(T >= 0 && H > 0 && V > 0, "zk_embed: bad sizes");
+  ZK_REQUIRE(!strip || H % 32 == 0, "zk_embed: strip layout needs H % 32 == 0");
   if (T == 0) return 0;
-  embed_kernel<act_t><<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)table, tokens, out, scale, H, V);
+  embed_kernel<act_t><<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)table, tokens, out, scale, H, V, strip);
   return zk_launch_status("zk_embed");
 }
 

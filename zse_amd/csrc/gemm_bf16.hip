@@ -49,16 +49,24 @@ template <int MT, bool GATED, int NW>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __restrict__ A, int lda,
                                                           const __bf16* __restrict__ W,
                                                           void* __restrict__ C, int ldc, int c_is_f32,
-                                                          int M, int N, int K, int epi, float cap) {
+                                                          int M, int N, int K, int epi, float cap,
+                                                          int w_strip) {
   constexpr int NS = GATED ? 2 : 1;
   __shared__ f32x4 red[NW - 1][NS][MT][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, kq = lane >> 4;
   const int n0 = blockIdx.x * 16;
+  // Row-major weights: a lane reads row n0 + r at 8 * kq, a 32-wide step further on is 32
+  // elements away.  Strip layout: the 64 lanes' pieces of one (strip, step) are one
+  // contiguous KB, a step further on is 512 elements away, strips follow each other.
   const int wrow = min(n0 + r, N - 1);
+  const int ksteps = (K + 31) / 32;
+  const size_t wstep = w_strip ? 512 : 32;
   const __bf16* wp[NS];
-  wp[0] = W + (size_t)wrow * K + kq * 8;
-  if (GATED) wp[NS - 1] = W + (size_t)(N + wrow) * K + kq * 8;
+  wp[0] = w_strip ? W + (size_t)blockIdx.x * ksteps * 512 + lane * 8 : W + (size_t)wrow * K + kq * 8;
+  if (GATED)
+    wp[NS - 1] = w_strip ? W + ((size_t)(N / 16) + blockIdx.x) * ksteps * 512 + lane * 8
+                         : W + (size_t)(N + wrow) * K + kq * 8;
   const __bf16* ap[MT];
   bool av[MT];
 #pragma unroll
@@ -88,7 +96,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) af[mt][s] = (in && av[mt]) ? *(const bf16x8*)(ap[mt] + k) : zero8();
 #pragma unroll
-      for (int g = 0; g < NS; g++) wf[g][s] = in ? *(const bf16x8*)(wp[g] + k) : zero8();
+      for (int g = 0; g < NS; g++) wf[g][s] = in ? *(const bf16x8*)(wp[g] + (size_t)(s0 + s) * wstep) : zero8();
     }
   };
   auto multiply = [&](const bf16x8 (&wf)[NS][STEPS], const bf16x8 (&af)[MT][STEPS]) {
@@ -157,7 +165,7 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
                                                         const __bf16* __restrict__ W,
                                                         void* __restrict__ C, int ldc, int c_is_f32,
                                                         int M, int N, int K, int epi, float cap,
-                                                        int tiles_m, int tiles_n) {
+                                                        int tiles_m, int tiles_n, int w_strip) {
   constexpr int BM = 64 * WMT;
   constexpr int APT = BM / 32;                 // 16-byte pieces of A a thread moves per k tile
   __shared__ __bf16 sA[BM][GT_LD];
@@ -180,14 +188,37 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
   const __bf16* gb[4];
 #pragma unroll
   for (int i = 0; i < APT; i++) ga[i] = A + (size_t)min(m0 + prow + 32 * i, M - 1) * lda + pcol;
+  int brow[4], bcol;      // where a thread's pieces of the weight tile land in LDS
+  if (w_strip) {
+    // a wave copies whole KB blocks: block (tid / 64) + 4 i of the tile's 8 strips x 2 steps,
+    // lane l = tid % 64 its 16 bytes; the k tile advances by two steps = 1024 elements
+    const int l = tid & 63, tstep = (tid >> 6) & 1;
+    const int ksteps = (K + 31) / 32;
+    const int strips = GATED ? 2 * N / 16 : (N + 15) / 16;
+    bcol = tstep * 32 + (l >> 4) * 8;
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int row = prow + 32 * i;
-    int bn;
-    if (GATED) bn = row < 64 ? min(n0 + row, N - 1) : N + min(n0 + row - 64, N - 1);
-    else bn = min(n0 + row, N - 1);
-    gb[i] = W + (size_t)bn * K + pcol;
+    for (int i = 0; i < 4; i++) {
+      const int sit = ((tid >> 6) + 4 * i) >> 1;            // strip within the tile
+      brow[i] = sit * 16 + (l & 15);
+      int gs;
+      if (GATED) gs = sit < 4 ? n0 / 16 + sit : N / 16 + n0 / 16 + (sit - 4);
+      else gs = n0 / 16 + sit;
+      gs = min(gs, strips - 1);
+      gb[i] = W + ((size_t)gs * ksteps + tstep) * 512 + l * 8;
+    }
+  } else {
+    bcol = pcol;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int row = prow + 32 * i;
+      brow[i] = row;
+      int bn;
+      if (GATED) bn = row < 64 ? min(n0 + row, N - 1) : N + min(n0 + row - 64, N - 1);
+      else bn = min(n0 + row, N - 1);
+      gb[i] = W + (size_t)bn * K + pcol;
+    }
   }
+  const size_t bstep = w_strip ? 1024 : GT_BK;      // elements between a piece and the same piece one k tile on
   f32x16 acc[WMT][2];
 #pragma unroll
   for (int i = 0; i < WMT; i++)
@@ -198,26 +229,26 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
 
   bf16x8 ra[APT], rb[4];
   {
-    const bool in = pcol < K;
+    const bool in = pcol < K, inb = bcol < K;
 #pragma unroll
     for (int i = 0; i < APT; i++) ra[i] = in ? *(const bf16x8*)(ga[i]) : zero8();
 #pragma unroll
-    for (int i = 0; i < 4; i++) rb[i] = in ? *(const bf16x8*)(gb[i]) : zero8();
+    for (int i = 0; i < 4; i++) rb[i] = inb ? *(const bf16x8*)(gb[i]) : zero8();
   }
   for (int k0 = 0; k0 < K; k0 += GT_BK) {
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < APT; i++) *(bf16x8*)(&sA[prow + 32 * i][pcol]) = ra[i];
 #pragma unroll
-    for (int i = 0; i < 4; i++) *(bf16x8*)(&sB[prow + 32 * i][pcol]) = rb[i];
+    for (int i = 0; i < 4; i++) *(bf16x8*)(&sB[brow[i]][bcol]) = rb[i];
     __syncthreads();
     const int kn = k0 + GT_BK;
     if (kn < K) {
-      const bool in = kn + pcol < K;
+      const bool in = kn + pcol < K, inb = kn + bcol < K;
 #pragma unroll
       for (int i = 0; i < APT; i++) ra[i] = in ? *(const bf16x8*)(ga[i] + kn) : zero8();
 #pragma unroll
-      for (int i = 0; i < 4; i++) rb[i] = in ? *(const bf16x8*)(gb[i] + kn) : zero8();
+      for (int i = 0; i < 4; i++) rb[i] = inb ? *(const bf16x8*)(gb[i] + (size_t)(kn / GT_BK) * bstep) : zero8();
     }
 #pragma unroll
     for (int ks = 0; ks < GT_BK / 16; ks++) {
@@ -271,14 +302,14 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
 
 template <bool GATED>
 static int launch_skinny(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M,
-                         int N, int K, int epi, float cap, hipStream_t s) {
+                         int N, int K, int epi, float cap, int w_strip, hipStream_t s) {
   const int mt = (M + 15) / 16;
   dim3 grid((N + 15) / 16);
   // few strips: eight waves a strip keep enough loads in flight
   const bool wide = grid.x < 512 && K >= 2048 && mt <= 2;
 #define ZK_SKINNY(MT_, NW_)                                                                           \
   gemm_skinny_kernel<MT_, GATED, NW_><<<grid, NW_ * 64, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, \
-                                                                C, ldc, c_is_f32, M, N, K, epi, cap)
+                                                                C, ldc, c_is_f32, M, N, K, epi, cap, w_strip)
   if (mt == 1) { if (wide) ZK_SKINNY(1, 8); else ZK_SKINNY(1, 4); }
   else if (mt == 2) { if (wide) ZK_SKINNY(2, 8); else ZK_SKINNY(2, 4); }
   else if (mt == 3) ZK_SKINNY(3, 4);
@@ -287,22 +318,53 @@ static int launch_skinny(const void* A, int lda, const void* W, void* C, int ldc
   return zk_launch_status("zk_gemm_bf16 (skinny)");
 }
 
+// Strip layout of a [N, K] weight matrix, K % 32 == 0: rows in strips of 16 (the last strip
+// padded with zeros), each (strip, 32-wide k step) one KB in which lane l = 16 * kq + r holds
+// W[16 * strip + r][32 * step + 8 * kq .. + 8], i.e. exactly what the 64 lanes of a wave load
+// for one 16x16x32 MFMA; steps follow each other, then strips.  A wave that streams its run
+// of steps reads contiguous memory instead of sixteen rows K elements apart, which keeps
+// every memory channel busy whatever K is (row strides of 4096 or 18432 bytes do not).
+__global__ void strip_layout_kernel(const __bf16* __restrict__ src, __bf16* __restrict__ dst, int N, int K,
+                                    size_t pieces) {
+  const size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (q >= pieces) return;
+  const int ksteps = K / 32;
+  const size_t block = q >> 6;
+  const int l = (int)(q & 63);
+  const int n = (int)(block / ksteps) * 16 + (l & 15);
+  const int k = (int)(block % ksteps) * 32 + (l >> 4) * 8;
+  *(bf16x8*)(dst + q * 8) = n < N ? *(const bf16x8*)(src + (size_t)n * K + k) : zero8();
+}
+
+// dst holds ceil(N / 16) * 16 rows of K elements.
+extern "C" int zk_strip_layout(const void* src, void* dst, int N, int K, void* stream) {
+  ZK_REQUIRE(N > 0 && K > 0 && K % 32 == 0, "zk_strip_layout: K must be a positive multiple of 32");
+  const size_t pieces = (size_t)((N + 15) / 16) * 16 * K / 8;
+  ZK_REQUIRE((pieces + 255) / 256 < 2147483647ull, "zk_strip_layout: matrix too large");
+  strip_layout_kernel<<<(unsigned)((pieces + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+      (const __bf16*)src, (__bf16*)dst, N, K, pieces);
+  return zk_launch_status("zk_strip_layout");
+}
+
 // epi: 0 none, 1 soft cap (cap > 0), 2 gelu_tanh gate, 3 silu gate.  For the gated
 // epilogues W is [2N, K] (gate rows, then up rows) and C is [M, N].
+// w_strip: W is in strip layout (zk_strip_layout), which needs K % 32 == 0 and, for the
+// gated epilogues, N % 16 == 0.
 extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
-                            int M, int N, int K, int epi, float cap, void* stream) {
+                            int M, int N, int K, int epi, float cap, int w_strip, void* stream) {
   ZK_REQUIRE(M >= 0 && N > 0 && K > 0, "zk_gemm_bf16: bad sizes");
   ZK_REQUIRE(K % 8 == 0 && lda % 8 == 0, "zk_gemm_bf16: K and lda must be multiples of 8");
   ZK_REQUIRE(lda >= K && ldc >= N, "zk_gemm_bf16: leading dimensions too small");
   ZK_REQUIRE(epi >= 0 && epi <= 3, "zk_gemm_bf16: unknown epilogue");
   ZK_REQUIRE(epi != EPI_SOFTCAP || cap > 0.f, "zk_gemm_bf16: soft cap must be positive");
   ZK_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "zk_gemm_bf16: operands must be 16-byte aligned");
+  const bool gated = epi >= EPI_GELU_TANH;
+  ZK_REQUIRE(!w_strip || (K % 32 == 0 && (!gated || N % 16 == 0)), "zk_gemm_bf16: strip layout needs K % 32 == 0 (and N % 16 == 0 when gated)");
   if (M == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
-  const bool gated = epi >= EPI_GELU_TANH;
   if (M <= 64) {
-    return gated ? launch_skinny<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, s)
-                 : launch_skinny<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, s);
+    return gated ? launch_skinny<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s)
+                 : launch_skinny<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s);
   }
   const int ncols = gated ? GT_BN / 2 : GT_BN;
   const int tiles_n = (N + ncols - 1) / ncols;
@@ -315,10 +377,10 @@ extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int 
   dim3 grid(tiles_m * tiles_n);
   if (gated)
     gemm_tile_kernel<2, true><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32,
-                                                   M, N, K, epi, cap, tiles_m, tiles_n);
+                                                   M, N, K, epi, cap, tiles_m, tiles_n, w_strip);
   else
     gemm_tile_kernel<2, false><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32,
-                                                    M, N, K, epi, cap, tiles_m, tiles_n);
+                                                    M, N, K, epi, cap, tiles_m, tiles_n, w_strip);
   return zk_launch_status("zk_gemm_bf16 (tile)");
 }
 

@@ -44,7 +44,7 @@ class Engine:
                  use_graphs: bool = True, quiet: bool = True):
         self.rt = Runtime.get(device_index)
         self.dtype = canonical_dtype(dtype)
-        self.model = load_model(model, self.dtype, self.rt) if isinstance(model, str) else model
+        self.model = load_model(model, self.dtype, self.rt, tuned=tuned) if isinstance(model, str) else model
         max_len = min(max_seq_len or self.model.plan.max_position, self.model.plan.max_position)
         if num_blocks is None:
             # enough for every request slot at a moderate length, bounded by memory left
@@ -58,7 +58,7 @@ class Engine:
         self.runner = StepRunner(self.model, self.rt, self.dtype, page_size=block_size,
                                  num_pages=num_blocks, max_seqs=max_batch_seqs,
                                  max_batch_tokens=max_batch_tokens, max_model_len=max_len,
-                                 tuned=tuned, use_graphs=use_graphs)
+                                 use_graphs=use_graphs)
         self.scheduler = Scheduler(SchedulerConfig(max_batch_tokens, prefill_chunk_size, max_batch_seqs),
                                    self.runner.manager)
         self.sampler = DeviceSampler(self.rt, self.runner.k, max_batch_seqs)

@@ -10,15 +10,18 @@ from ..weights.loader import CheckpointWeights, RandomWeights
 from .model import Model
 
 
-def load_model(model_dir: str, dtype: str, rt: Optional[Runtime] = None) -> Model:
-    """Read config.json, pick the architecture, check and load the safetensors."""
+def load_model(model_dir: str, dtype: str, rt: Optional[Runtime] = None, tuned: bool = True) -> Model:
+    """Read config.json, pick the architecture, check and load the safetensors.  ``tuned``:
+    the model will run on the tuned kernels (weights may then sit in their layouts); False
+    keeps everything row-major for the plain kernels."""
     rt = rt or Runtime.get()
     dtype = canonical_dtype(dtype)
     arch, config = load_config(model_dir)
     model = Model(arch.plan(config))
     model.config = config
-    src = CheckpointWeights(rt, dtype, model_dir, model.tensor_reqs(), model.plan.ignored_tensors)
+    src = CheckpointWeights(rt, dtype, model_dir, model.tensor_reqs(), model.plan.ignored_tensors, tuned=tuned)
     model.load(src, rt, dtype)
+    model.tuned = bool(tuned)
     rt.sync()
     model.weight_bytes = src.bytes_on_device
     src.close()
@@ -26,7 +29,7 @@ def load_model(model_dir: str, dtype: str, rt: Optional[Runtime] = None) -> Mode
 
 
 def random_model(config: dict, dtype: str, seed: int = 0, std: float = 0.02, gain_std: float = 0.1,
-                 rt: Optional[Runtime] = None) -> Model:
+                 rt: Optional[Runtime] = None, tuned: bool = True) -> Model:
     """A model with seeded random weights made on the device (no folder is written)."""
     rt = rt or Runtime.get()
     dtype = canonical_dtype(dtype)
@@ -34,8 +37,9 @@ def random_model(config: dict, dtype: str, seed: int = 0, std: float = 0.02, gai
     typed = arch.config_from_dict(config)
     model = Model(arch.plan(typed))
     model.config = typed
-    src = RandomWeights(rt, dtype, model.tensor_reqs(), seed, std, gain_std)
+    src = RandomWeights(rt, dtype, model.tensor_reqs(), seed, std, gain_std, tuned=tuned)
     model.load(src, rt, dtype)
+    model.tuned = bool(tuned)
     rt.sync()
     model.weight_bytes = src.bytes_on_device
     return model

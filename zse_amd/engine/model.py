@@ -36,6 +36,7 @@ class Model:
                 raise ValueError(f"order entry {i} reads the cache of entry {call.cache_of}, "
                                  f"which does not run before it")
         self.loaded_dtype: Optional[str] = None
+        self.tuned = True            # set at load: whether weights may sit in the tuned kernels' layouts
 
     def parts(self) -> List[Part]:
         out = []

@@ -59,11 +59,11 @@ def main(argv: Optional[list] = None) -> int:
 
     print(f"[trace_run] loading {a.model} as {a.dtype}", file=sys.stderr, flush=True)
     rt = Runtime.get()
-    model = load_model(a.model, a.dtype, rt)
+    model = load_model(a.model, a.dtype, rt, tuned=not a.plain)
     max_len = min(model.plan.max_position, max(a.max_tokens, 64))
     runner = StepRunner(model, rt, a.dtype, page_size=a.block_size, cache_tokens=a.max_tokens,
                         max_seqs=a.max_seqs, max_batch_tokens=max(a.max_tokens, 64),
-                        max_model_len=max_len, tuned=not a.plain, use_graphs=False)
+                        max_model_len=max_len, use_graphs=False)
     print(f"[trace_run] ready: {model.plan.architecture}, {len(model.plan.order)} layer calls, "
           f"pages of {a.block_size}", file=sys.stderr, flush=True)
     replay(runner, sys.stdin, a.out, log=sys.stdout)

@@ -126,13 +126,16 @@ class StepRunner:
     def __init__(self, model: Model, rt: Runtime, dtype: str, page_size: int = 16,
                  num_pages: Optional[int] = None, cache_tokens: Optional[int] = None,
                  max_seqs: int = 64, max_batch_tokens: int = 4096, max_model_len: Optional[int] = None,
-                 tuned: bool = True, use_graphs: bool = True):
+                 tuned: Optional[bool] = None, use_graphs: bool = True):
         self.model, self.rt = model, rt
         self.dtype = canonical_dtype(dtype)
         if model.loaded_dtype != self.dtype:
             raise ValueError(f"the model's weights are {model.loaded_dtype}, the runner wants {self.dtype}")
         self.k = rt.kernels(self.dtype)
-        self.tuned = bool(tuned)
+        model_tuned = bool(getattr(model, "tuned", True))
+        if tuned is not None and bool(tuned) != model_tuned:
+            raise ValueError(f"the model was loaded with tuned={model_tuned}; the runner cannot run it with tuned={tuned}")
+        self.tuned = model_tuned
         self.use_graphs = bool(use_graphs) and self.tuned
         self.page_size = int(page_size)
         self.max_seqs = int(max_seqs)

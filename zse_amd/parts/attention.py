@@ -46,8 +46,11 @@ class PagedAttention(Part):
     def load(self, weights, rt, dtype):
         s = self.spec
         names = [s.names["q"]] if self.shared_kv else [s.names[r] for r in ("q", "k", "v")]
-        self.w_qkv = weights.matrix(names)
-        self.w_o = weights.matrix([s.names["o"]])
+        strip = getattr(weights, "wants_strip", None)
+        self.w_qkv = weights.matrix(names, strip=True) if strip and strip(s.hidden_size) else weights.matrix(names)
+        o_cols = s.num_heads * s.head_dim
+        self.w_o = (weights.matrix([s.names["o"]], strip=True) if strip and strip(o_cols)
+                    else weights.matrix([s.names["o"]]))
 
     def cache_need(self):
         s = self.spec

@@ -28,7 +28,10 @@ class Embedding(Part):
         return [TensorReq(self.spec.weight, (self.spec.vocab_size, self.spec.hidden_size))]
 
     def load(self, weights, rt, dtype):
-        self.table = weights.matrix([self.spec.weight])
+        # the table may be the head's matrix too (tied): both ask for the same layout
+        strip = getattr(weights, "wants_strip", None)
+        self.table = (weights.matrix([self.spec.weight], strip=True) if strip and strip(self.spec.hidden_size)
+                      else weights.matrix([self.spec.weight]))
         # the scalar is kept in the table's storage type, as the reference keeps its own
         # (model_runner.py:155-158); the product is float
         s = np.float32(self.spec.scale)
@@ -41,7 +44,7 @@ class Embedding(Part):
         s = self.spec
         h = ctx.alloc((ctx.T, s.hidden_size), F32)
         ctx.k.zk_embed(self.table.ptr, ctx.tokens, h.ptr, self.scale, ctx.T, s.hidden_size,
-                       s.vocab_size, ctx.stream)
+                       s.vocab_size, 1 if self.table.layout == "strip" else 0, ctx.stream)
         return h
 
 
@@ -54,7 +57,9 @@ class LMHead(Part):
         return [TensorReq(self.spec.weight, (self.spec.vocab_size, self.spec.hidden_size))]
 
     def load(self, weights, rt, dtype):
-        self.weight = weights.matrix([self.spec.weight])
+        strip = getattr(weights, "wants_strip", None)
+        self.weight = (weights.matrix([self.spec.weight], strip=True) if strip and strip(self.spec.hidden_size)
+                       else weights.matrix([self.spec.weight]))
 
     def forward(self, ctx, x: Tensor, out: Tensor) -> Tensor:
         """x: normed rows [K, hidden]; out: float logits [K, vocab]."""

@@ -31,8 +31,12 @@ class GatedMLP(Part):
 
     def load(self, weights, rt, dtype):
         s = self.spec
-        self.w_gu = weights.matrix([s.names["gate"], s.names["up"]])
-        self.w_down = weights.matrix([s.names["down"]])
+        strip = getattr(weights, "wants_strip", None)
+        gu = [s.names["gate"], s.names["up"]]
+        self.w_gu = (weights.matrix(gu, strip=True) if strip and strip(s.hidden_size, s.intermediate_size)
+                     else weights.matrix(gu))
+        self.w_down = (weights.matrix([s.names["down"]], strip=True) if strip and strip(s.intermediate_size)
+                       else weights.matrix([s.names["down"]]))
 
     def forward(self, ctx, x: Tensor) -> Tensor:
         s = self.spec

@@ -37,9 +37,12 @@ def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0
         raise ValueError(f"linear: out must be float32 or {ctx.dtype}, got {out.dtype}")
     out_f32 = 1 if out.dtype == F32 else 0
     k = ctx.k
+    strip = w.layout == "strip"
+    if strip and not tuned_gemm(ctx, K):
+        raise ValueError("linear: weights in strip layout need the matrix-core product")
     if tuned_gemm(ctx, K):
         k.zk_gemm_bf16(x.ptr, K, w.ptr, out.ptr, N, out_f32, M, N, K, EPILOGUES[epilogue], float(cap),
-                       ctx.stream)
+                       1 if strip else 0, ctx.stream)
     else:
         k.zk_gemm_plain(x.ptr, K, w.ptr, out.ptr, N, out_f32, M, N, K, ctx.stream)
     return out

@@ -38,13 +38,14 @@ class DeviceError(RuntimeError):
 class Tensor:
     """A view of device memory: pointer, shape, dtype.  Row-major, contiguous."""
 
-    __slots__ = ("ptr", "shape", "dtype", "owner")
+    __slots__ = ("ptr", "shape", "dtype", "owner", "layout")
 
-    def __init__(self, ptr: int, shape: Sequence[int], dtype: str, owner=None):
+    def __init__(self, ptr: int, shape: Sequence[int], dtype: str, owner=None, layout: str = "rows"):
         self.ptr = int(ptr)
         self.shape = tuple(int(s) for s in shape)
         self.dtype = dtype
         self.owner = owner      # keeps the allocation alive
+        self.layout = layout    # "rows": row-major; "strip": the matrix-core kernels' weight layout
 
     @property
     def numel(self) -> int:
@@ -140,7 +141,7 @@ _VP, _I, _F, _SZ, _U64 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint64
 
 # name -> argument types (all return int; 0 = success)
 KERNEL_SIGNATURES = {
-    "zk_embed": [_VP, _VP, _VP, _F, _I, _I, _I, _VP],
+    "zk_embed": [_VP, _VP, _VP, _F, _I, _I, _I, _I, _VP],
     "zk_rmsnorm": [_VP, _I, _VP, _VP, _VP, _F, _I, _I, _I, _VP],
     "zk_norm_add_norm": [_VP, _VP, _F, _I, _VP, _VP, _F, _I, _VP, _I, _I, _VP],
     "zk_gated_act": [_VP, _VP, _I, _I, _I, _VP],
@@ -157,7 +158,8 @@ KERNEL_SIGNATURES = {
 }
 # present only in the bf16 library
 BF16_KERNEL_SIGNATURES = {
-    "zk_gemm_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _VP],
+    "zk_gemm_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
+    "zk_strip_layout": [_VP, _VP, _I, _I, _VP],
     "zk_attention_bf16": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
                           _F, _F, _I, _VP, _SZ, _VP],
 }

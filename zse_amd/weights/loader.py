@@ -90,16 +90,35 @@ def check_folder(model_dir: str, reqs: Iterable[TensorReq], ignored: Sequence[st
 class _Source:
     """Common part of weight sources: caching, so that tied names share one tensor."""
 
-    def __init__(self, rt, dtype: str):
+    def __init__(self, rt, dtype: str, tuned: bool = True):
         self.rt = rt
         self.dtype = dtype
+        self.tuned = bool(tuned)      # parts may ask for layouts that only the tuned kernels read
         self.k = rt.kernels(dtype)
         self._cache: Dict[Tuple, Tensor] = {}
         self.bytes_on_device = 0
 
-    def matrix(self, names: Sequence[str]) -> Tensor:
-        """The named 2-D tensors stacked along rows, in the compute type."""
-        key = ("m",) + tuple(_strip(n) for n in names)
+    def wants_strip(self, cols: int, gated_rows: int = 0) -> bool:
+        """True when a matrix with ``cols`` columns should be held in the matrix-core kernels'
+        strip layout: bf16, tuned kernels on, whole 32-wide steps (and, for a gate|up stack
+        of ``gated_rows`` each, whole strips of 16)."""
+        return bool(self.tuned and self.dtype == BF16 and self.k.has("zk_strip_layout") and
+                    cols % 32 == 0 and gated_rows % 16 == 0)
+
+    def matrix(self, names: Sequence[str], strip: bool = False) -> Tensor:
+        """The named 2-D tensors stacked along rows, in the compute type.  ``strip``: in strip
+        layout (rows padded to a multiple of 16; the shape stays the logical one)."""
+        key = ("s" if strip else "m",) + tuple(_strip(n) for n in names)
+        if key not in self._cache and strip:
+            rows = self.matrix(names)
+            self._cache.pop(("m",) + tuple(_strip(n) for n in names))
+            self.bytes_on_device -= rows.nbytes
+            n, k = rows.shape
+            out = self.rt.empty(((n + 15) // 16 * 16, k), self.dtype)
+            self.k.zk_strip_layout(rows.ptr, out.ptr, n, k, self.rt.stream)
+            self.rt.sync()
+            self.bytes_on_device += out.nbytes
+            self._cache[key] = Tensor(out.ptr, (n, k), self.dtype, out.owner, layout="strip")
         if key not in self._cache:
             shapes = [self._shape(n) for n in names]
             cols = shapes[0][1]
@@ -128,8 +147,8 @@ class CheckpointWeights(_Source):
     """Tensors of a checked model folder, copied and converted on the device."""
 
     def __init__(self, rt, dtype: str, model_dir: str, reqs: Iterable[TensorReq],
-                 ignored: Sequence[str] = ()):
-        super().__init__(rt, dtype)
+                 ignored: Sequence[str] = (), tuned: bool = True):
+        super().__init__(rt, dtype, tuned)
         self.entries = check_folder(model_dir, reqs, ignored)
         self._staging = None
 
@@ -168,8 +187,8 @@ class RandomWeights(_Source):
     N(0, gain_std); each value is a function of (seed, tensor name, index)."""
 
     def __init__(self, rt, dtype: str, reqs: Iterable[TensorReq], seed: int, std: float = 0.02,
-                 gain_std: float = 0.1):
-        super().__init__(rt, dtype)
+                 gain_std: float = 0.1, tuned: bool = True):
+        super().__init__(rt, dtype, tuned)
         self.reqs = merge_reqs(reqs)
         self.seed, self.std, self.gain_std = int(seed), float(std), float(gain_std)
 
