@@ -34,6 +34,16 @@ def _drop_device_tensors():
     _ALIVE.clear()
 
 
+_GEMM_WS = {}
+
+
+def gemm_workspace(rt):
+    """One workspace for the split products, as the engine keeps one."""
+    if "ws" not in _GEMM_WS:
+        _GEMM_WS["ws"] = rt.zeros((rt.kernels("bfloat16").zk_gemm_bf16_workspace() // 4,), "float32")
+    return _GEMM_WS["ws"]
+
+
 def ptr(t):
     """A tensor's device pointer; the tensor stays allocated until the test ends (a kernel
     that was only enqueued must not find its operand freed)."""
@@ -73,13 +83,13 @@ def test_gemm_bf16_matrix_cores(rt, M, N, K):
     A, W = up(rt, a, "bfloat16"), up(rt, w, "bfloat16")
     want = a.astype(np.float64) @ w.astype(np.float64).T
     C = rt.empty((M, N), "float32")
-    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, N, 1, M, N, K, 0, 0.0, 0, rt.stream)
+    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, N, 1, M, N, K, 0, 0.0, 0, None, 0, rt.stream)
     assert np.abs(rt.download(C) - want).max() < 1e-4 * math.sqrt(K)      # float accumulation
     Cb = rt.empty((M, N), "bfloat16")
-    k.zk_gemm_bf16(A.ptr, K, W.ptr, Cb.ptr, N, 0, M, N, K, 0, 0.0, 0, rt.stream)
+    k.zk_gemm_bf16(A.ptr, K, W.ptr, Cb.ptr, N, 0, M, N, K, 0, 0.0, 0, None, 0, rt.stream)
     got = rt.download_f32(Cb)
     assert np.abs(got - want).max() <= np.abs(want).max() * 2.0 ** -8 + 1e-4 * math.sqrt(K)
-    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, N, 1, M, N, K, 1, 7.5, 0, rt.stream)
+    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, N, 1, M, N, K, 1, 7.5, 0, None, 0, rt.stream)
     assert np.abs(rt.download(C) - 7.5 * np.tanh(want / 7.5)).max() < 1e-4 * math.sqrt(K)
 
 
@@ -91,7 +101,7 @@ def test_gemm_bf16_gated_epilogue(rt, M, I, K, act):
     a, w = bf16(rng.normal(size=(M, K))), bf16(rng.normal(size=(2 * I, K)) * 0.3)
     A, W = up(rt, a, "bfloat16"), up(rt, w, "bfloat16")
     C = rt.empty((M, I), "float32")
-    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, I, 1, M, I, K, 2 if act == "gelu_tanh" else 3, 0.0, 0, rt.stream)
+    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, I, 1, M, I, K, 2 if act == "gelu_tanh" else 3, 0.0, 0, None, 0, rt.stream)
     g = a.astype(np.float64) @ w[:I].astype(np.float64).T
     u = a.astype(np.float64) @ w[I:].astype(np.float64).T
     want = (gelu(g) if act == "gelu_tanh" else g / (1 + np.exp(-g))) * u
@@ -100,7 +110,11 @@ def test_gemm_bf16_gated_epilogue(rt, M, I, K, act):
 
 @pytest.mark.parametrize("M,N,K,gated", [(1, 1000, 96, False), (8, 2304, 2048, False), (40, 50, 64, False),
                                           (64, 333, 320, False), (200, 1000, 320, False), (300, 257, 2304, False),
-                                          (3, 176, 64, True), (16, 320, 96, True), (130, 336, 128, True)])
+                                          (3, 176, 64, True), (16, 320, 96, True), (130, 336, 128, True),
+                                          # 17..64 rows: activations shared in LDS, one to eight k chunks
+                                          (17, 100, 64, False), (33, 2304, 2048, False), (48, 333, 544, False),
+                                          (64, 1000, 512, False), (50, 72, 800, False), (20, 176, 288, True),
+                                          (64, 320, 800, True), (40, 336, 256, True), (33, 48, 1056, True)])
 def test_gemm_bf16_strip_layout(rt, M, N, K, gated):
     """The same products with the weights rearranged into strips of 16 rows by 32 columns, and
     an embedding gather out of that layout."""
@@ -112,16 +126,24 @@ def test_gemm_bf16_strip_layout(rt, M, N, K, gated):
     WS = rt.empty(((rows + 15) // 16 * 16, K), "bfloat16")
     k.zk_strip_layout(W.ptr, WS.ptr, rows, K, rt.stream)
     C = rt.empty((M, N), "float32")
+    ws = gemm_workspace(rt)
     if gated:
-        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 2, 0.0, 1, rt.stream)
+        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 2, 0.0, 1, ws.ptr, ws.nbytes, rt.stream)
         g = a.astype(np.float64) @ w[:N].astype(np.float64).T
         want = gelu(g) * (a.astype(np.float64) @ w[N:].astype(np.float64).T)
         tol = 2e-4 * math.sqrt(K) * max(1.0, np.abs(want).max())
     else:
-        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 0, 0.0, 1, rt.stream)
+        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 0, 0.0, 1, ws.ptr, ws.nbytes, rt.stream)
         want = a.astype(np.float64) @ w.astype(np.float64).T
         tol = 1e-4 * math.sqrt(K)
-    assert np.abs(rt.download(C) - want).max() < tol
+    got = rt.download(C)
+    assert np.abs(got - want).max() < tol
+    # a second launch, over the first one's leavings in the workspace, gives the same bits
+    k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 2 if gated else 0, 0.0, 1, ws.ptr, ws.nbytes, rt.stream)
+    assert np.array_equal(rt.download(C), got)
+    if 16 < M <= 64:   # without a workspace K is not split over blocks: same values beyond rounding
+        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 2 if gated else 0, 0.0, 1, None, 0, rt.stream)
+        assert np.abs(rt.download(C) - want).max() < tol
     if not gated and K % 32 == 0:
         toks = rng.integers(0, N, 5).astype(np.int32)
         toks[0] = N - 1
@@ -145,7 +167,7 @@ def test_gemm_refuses_what_it_cannot_do(rt):
     k = rt.kernels("bfloat16")
     A, W, C = rt.empty((4, 100), "bfloat16"), rt.empty((8, 100), "bfloat16"), rt.empty((4, 8), "float32")
     with pytest.raises(DeviceError, match="multiples of 8"):
-        k.zk_gemm_bf16(A.ptr, 100, W.ptr, C.ptr, 8, 1, 4, 8, 100, 0, 0.0, 0, rt.stream)
+        k.zk_gemm_bf16(A.ptr, 100, W.ptr, C.ptr, 8, 1, 4, 8, 100, 0, 0.0, 0, None, 0, rt.stream)
 
 
 # ------------------------------------------------------------------ attention over the cache

@@ -33,6 +33,7 @@ class Ctx:
         self.rt, self.k, self.dtype, self.tuned, self.stream = rt, rt.kernels(dtype), dtype, tuned, rt.stream
         self.arena = Arena(rt, 1 << 20)
         self.workspace = rt.zeros((1 << 16,), "float32")
+        self.gemm_workspace = None
 
     def alloc(self, shape, dtype=None):
         return self.arena.alloc(shape, dtype or self.dtype)

@@ -300,6 +300,192 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
 }
 
 
+// ------------------------------------------------------------------ mid (16 < M <= 64)
+// With more than one column tile the activations weigh more than the weights on the way
+// from L2 to the CUs when every 16-row strip fetches them again (64 rows of A per 16 rows
+// of W).  Here a block owns four strips, one per wave, all four walk K together, and the
+// activations of the current 256-wide k chunk wait in LDS for all of them: 64 rows of A per
+// 64 rows of W.  Weights come straight from global memory in strip layout, the next chunk's
+// loads are in flight while the current one is multiplied.
+//
+// Few column blocks (N of a few thousand) cannot fill 256 CUs, so blockIdx.y splits K into
+// `ksplit` ranges.  Then each block leaves its partial sums in the workspace and a second,
+// small kernel adds them in the order of the ranges and applies the epilogue.  (One kernel
+// with a ticket per column block, the last block adding up, was measured three times slower:
+// the device-wide fences it needs write back and invalidate the L2 of every XCD.)
+#define GM_STEPS 8
+#define GM_LD (GM_STEPS * 32 + 8)
+
+// A lane's results of one strip: rows n = 16 * strip + 4 * kq + i of W, column m = 16 * mt + r of A.
+template <int MT, bool GATED>
+__device__ __forceinline__ void mid_store(const f32x4 (&acc)[GATED ? 2 : 1][MT], void* __restrict__ C, int ldc,
+                                          int c_is_f32, int M, int N, int strip, int lane, int epi, float cap) {
+  const int r = lane & 15, kq = lane >> 4;
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) {
+    const int m = mt * 16 + r;
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int n = strip * 16 + 4 * kq + i;
+      if (n >= N) continue;
+      float x = acc[0][mt][i];
+      if (GATED) x = epi_gate(x, acc[GATED ? 1 : 0][mt][i], epi);
+      else if (epi == EPI_SOFTCAP) x = cap * tanhf(x / cap);
+      if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
+      else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
+    }
+  }
+}
+
+template <int MT, bool GATED>
+__global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict__ A, int lda,
+                                                       const __bf16* __restrict__ W,
+                                                       void* __restrict__ C, int ldc, int c_is_f32,
+                                                       int M, int N, int K, int epi, float cap,
+                                                       f32x4* __restrict__ partials, int ksplit) {
+  constexpr int NS = GATED ? 2 : 1;
+  __shared__ __bf16 sA[2][MT * 16][GM_LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, kq = lane >> 4;
+  const int ksteps = K / 32;
+  const int s_begin = (int)((long)blockIdx.y * ksteps / ksplit);
+  const int s_end = (int)((long)(blockIdx.y + 1) * ksteps / ksplit);
+  const int nstrips = (N + 15) / 16;
+  const int strip = blockIdx.x * 4 + wave;
+  const bool strip_ok = strip < nstrips;
+  const __bf16* wp[NS];
+  wp[0] = W + (size_t)(strip_ok ? strip : 0) * ksteps * 512 + lane * 8;
+  if (GATED) wp[NS - 1] = W + ((size_t)(N / 16) + (strip_ok ? strip : 0)) * ksteps * 512 + lane * 8;
+  // A pieces of a chunk: MT*16 rows x 32 pieces of 16 bytes; a wave reads two rows' 512 contiguous bytes
+  constexpr int APT = MT * 16 * 32 / 256;
+  const int a_piece = tid & 31, a_row0 = tid >> 5;     // rows a_row0 + 8 j
+  f32x4 acc[NS][MT];
+#pragma unroll
+  for (int g = 0; g < NS; g++)
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) acc[g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  auto fetch_a = [&](int s0, bf16x8 (&ra)[APT]) {
+#pragma unroll
+    for (int j = 0; j < APT; j++) {
+      const int row = a_row0 + 8 * j;
+      const int k = s0 * 32 + a_piece * 8;
+      ra[j] = (row < M && s0 + a_piece / 4 < s_end) ? *(const bf16x8*)(A + (size_t)row * lda + k) : zero8();
+    }
+  };
+  auto stash_a = [&](int buf, const bf16x8 (&ra)[APT]) {
+#pragma unroll
+    for (int j = 0; j < APT; j++) *(bf16x8*)(&sA[buf][a_row0 + 8 * j][a_piece * 8]) = ra[j];
+  };
+  auto fetch_w = [&](int s0, bf16x8 (&wf)[NS][GM_STEPS]) {
+#pragma unroll
+    for (int s = 0; s < GM_STEPS; s++)
+#pragma unroll
+      for (int g = 0; g < NS; g++)
+        wf[g][s] = (strip_ok && s0 + s < s_end) ? *(const bf16x8*)(wp[g] + (size_t)(s0 + s) * 512) : zero8();
+  };
+  auto multiply = [&](int buf, const bf16x8 (&wf)[NS][GM_STEPS]) {
+#pragma unroll
+    for (int s = 0; s < GM_STEPS; s++)
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) {
+        const bf16x8 af = *(const bf16x8*)(&sA[buf][mt * 16 + r][s * 32 + kq * 8]);
+#pragma unroll
+        for (int g = 0; g < NS; g++)
+          acc[g][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][s], af, acc[g][mt], 0, 0, 0);
+      }
+  };
+
+  bf16x8 ra[APT], w0[NS][GM_STEPS], w1[NS][GM_STEPS];
+  fetch_a(s_begin, ra);
+  fetch_w(s_begin, w0);
+  stash_a(0, ra);
+  __syncthreads();
+  for (int s0 = s_begin; s0 < s_end; s0 += 2 * GM_STEPS) {
+    const bool more1 = s0 + GM_STEPS < s_end;
+    if (more1) {
+      fetch_a(s0 + GM_STEPS, ra);
+      fetch_w(s0 + GM_STEPS, w1);
+    }
+    multiply(0, w0);
+    if (!more1) break;
+    stash_a(1, ra);
+    __syncthreads();
+    const bool more2 = s0 + 2 * GM_STEPS < s_end;
+    if (more2) {
+      fetch_a(s0 + 2 * GM_STEPS, ra);
+      fetch_w(s0 + 2 * GM_STEPS, w0);
+    }
+    multiply(1, w1);
+    if (!more2) break;
+    stash_a(0, ra);
+    __syncthreads();
+  }
+  if (ksplit > 1) {
+    if (!strip_ok) return;
+    f32x4* mine = partials + (((size_t)blockIdx.x * ksplit + blockIdx.y) * 4 + wave) * (NS * MT * 64) + lane;
+#pragma unroll
+    for (int g = 0; g < NS; g++)
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) mine[(g * MT + mt) * 64] = acc[g][mt];
+    return;
+  }
+  if (strip_ok) mid_store<MT, GATED>(acc, C, ldc, c_is_f32, M, N, strip, lane, epi, cap);
+}
+
+// Second half of a product whose K was split over blocks: the partial sums of a column block,
+// added in the order of the ranges, then the epilogue.  Same lanes, same values per lane as in
+// the product kernel.
+template <int MT, bool GATED>
+__global__ __launch_bounds__(256) void gemm_mid_join_kernel(const f32x4* __restrict__ partials, int ksplit,
+                                                            void* __restrict__ C, int ldc, int c_is_f32,
+                                                            int M, int N, int epi, float cap) {
+  constexpr int NS = GATED ? 2 : 1;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int strip = blockIdx.x * 4 + wave;
+  if (strip >= (N + 15) / 16) return;
+  const f32x4* all = partials + (((size_t)blockIdx.x * ksplit) * 4 + wave) * (NS * MT * 64) + lane;
+  f32x4 acc[NS][MT];
+#pragma unroll
+  for (int g = 0; g < NS; g++)
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) acc[g][mt] = all[(g * MT + mt) * 64];
+  for (int p = 1; p < ksplit; p++)
+#pragma unroll
+    for (int g = 0; g < NS; g++)
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) acc[g][mt] += all[((size_t)p * 4 * NS * MT + g * MT + mt) * 64];
+  mid_store<MT, GATED>(acc, C, ldc, c_is_f32, M, N, strip, lane, epi, cap);
+}
+
+template <bool GATED>
+static int launch_mid(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M, int N,
+                      int K, int epi, float cap, void* ws, size_t ws_bytes, hipStream_t s) {
+  const int mt = (M + 15) / 16;
+  const int cblocks = ((N + 15) / 16 + 3) / 4;
+  // split K until every CU has a block, a range no shorter than a chunk; more ranges than that
+  // cost more in partial sums than they gain (measured at N = 2304 and 4096, M = 32 and 64)
+  int ksplit = 256 / cblocks;
+  if (ksplit > K / 32 / GM_STEPS) ksplit = K / 32 / GM_STEPS;
+  if (ksplit < 1) ksplit = 1;
+  const size_t per_range = (size_t)4 * (GATED ? 2 : 1) * mt * 64 * sizeof(f32x4);
+  if (ws == nullptr || (uintptr_t)ws % 16 != 0) ksplit = 1;
+  while (ksplit > 1 && (size_t)cblocks * ksplit * per_range > ws_bytes) ksplit--;
+  f32x4* partials = (f32x4*)ws;
+  dim3 grid(cblocks, ksplit);
+#define ZK_MID(MT_)                                                                                   \
+  gemm_mid_kernel<MT_, GATED><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, \
+                                                   M, N, K, epi, cap, partials, ksplit);                \
+  if (ksplit > 1)                                                                                     \
+    gemm_mid_join_kernel<MT_, GATED><<<cblocks, 256, 0, s>>>(partials, ksplit, C, ldc, c_is_f32, M, N, epi, cap)
+  if (mt == 2) { ZK_MID(2); }
+  else if (mt == 3) { ZK_MID(3); }
+  else { ZK_MID(4); }
+#undef ZK_MID
+  return zk_launch_status("zk_gemm_bf16 (mid)");
+}
+
 template <bool GATED>
 static int launch_skinny(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M,
                          int N, int K, int epi, float cap, int w_strip, hipStream_t s) {
@@ -350,8 +536,13 @@ extern "C" int zk_strip_layout(const void* src, void* dst, int N, int K, void* s
 // epilogues W is [2N, K] (gate rows, then up rows) and C is [M, N].
 // w_strip: W is in strip layout (zk_strip_layout), which needs K % 32 == 0 and, for the
 // gated epilogues, N % 16 == 0.
+// The workspace may be null; then K is never split over blocks.  It holds nothing between
+// launches and serves one launch at a time.
+extern "C" size_t zk_gemm_bf16_workspace() { return (size_t)16 << 20; }
+
 extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
-                            int M, int N, int K, int epi, float cap, int w_strip, void* stream) {
+                            int M, int N, int K, int epi, float cap, int w_strip, void* ws,
+                            size_t ws_bytes, void* stream) {
   ZK_REQUIRE(M >= 0 && N > 0 && K > 0, "zk_gemm_bf16: bad sizes");
   ZK_REQUIRE(K % 8 == 0 && lda % 8 == 0, "zk_gemm_bf16: K and lda must be multiples of 8");
   ZK_REQUIRE(lda >= K && ldc >= N, "zk_gemm_bf16: leading dimensions too small");
@@ -362,6 +553,10 @@ extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int 
   ZK_REQUIRE(!w_strip || (K % 32 == 0 && (!gated || N % 16 == 0)), "zk_gemm_bf16: strip layout needs K % 32 == 0 (and N % 16 == 0 when gated)");
   if (M == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  if (M > 16 && M <= 64 && w_strip) {
+    return gated ? launch_mid<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, ws, ws_bytes, s)
+                 : launch_mid<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, ws, ws_bytes, s);
+  }
   if (M <= 64) {
     return gated ? launch_skinny<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s)
                  : launch_skinny<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s);

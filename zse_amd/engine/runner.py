@@ -103,6 +103,7 @@ class StepContext:
         self.stream = runner.rt.stream
         self.arena = runner.arena
         self.workspace = runner.workspace
+        self.gemm_workspace = runner.gemm_workspace
         self.T = 0
         self.R = 0
         self.tokens = self.positions = self.req_of_token = self.q_start = self.ctx_len = 0
@@ -182,6 +183,9 @@ class StepRunner:
         # ---- step buffers
         self.arena = Arena(rt)
         self.workspace = rt.zeros((self._workspace_words(),), F32)
+        self.gemm_workspace = None
+        if self.dtype == BF16 and self.k.has("zk_gemm_bf16_workspace"):
+            self.gemm_workspace = rt.zeros((self.k.zk_gemm_bf16_workspace() // 4,), F32)
         G = len(groups)
         self.max_blocks = self.manager.max_blocks
         cap = self._meta_words(self.max_batch_tokens, self.max_seqs, G)

@@ -41,8 +41,10 @@ def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0
     if strip and not tuned_gemm(ctx, K):
         raise ValueError("linear: weights in strip layout need the matrix-core product")
     if tuned_gemm(ctx, K):
+        ws = getattr(ctx, "gemm_workspace", None)      # lets a product of few columns split K over blocks
         k.zk_gemm_bf16(x.ptr, K, w.ptr, out.ptr, N, out_f32, M, N, K, EPILOGUES[epilogue], float(cap),
-                       1 if strip else 0, ctx.stream)
+                       1 if strip else 0, ws.ptr if ws is not None else None,
+                       ws.nbytes if ws is not None else 0, ctx.stream)
     else:
         k.zk_gemm_plain(x.ptr, K, w.ptr, out.ptr, N, out_f32, M, N, K, ctx.stream)
     return out

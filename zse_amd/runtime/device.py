@@ -158,7 +158,7 @@ KERNEL_SIGNATURES = {
 }
 # present only in the bf16 library
 BF16_KERNEL_SIGNATURES = {
-    "zk_gemm_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
+    "zk_gemm_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, C.c_size_t, _VP],
     "zk_strip_layout": [_VP, _VP, _I, _I, _VP],
     "zk_attention_bf16": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
                           _F, _F, _I, _VP, _SZ, _VP],
@@ -191,6 +191,9 @@ class KernelLibrary:
             self._dll.zk_attention_bf16_workspace.restype = C.c_size_t
             self._dll.zk_attention_bf16_workspace.argtypes = [_I, _I, _I, _I]
             self.zk_attention_bf16_workspace = self._dll.zk_attention_bf16_workspace
+            self._dll.zk_gemm_bf16_workspace.restype = C.c_size_t
+            self._dll.zk_gemm_bf16_workspace.argtypes = []
+            self.zk_gemm_bf16_workspace = self._dll.zk_gemm_bf16_workspace
         want = 1 if dtype == BF16 else 0
         if self._dll.zk_act_is_bf16() != want:
             raise DeviceError(f"{path} was built for the other storage type")
