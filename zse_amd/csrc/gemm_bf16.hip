@@ -151,74 +151,74 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
 }
 
 // ------------------------------------------------------------------ tile
-// Block tile (64 * WMT) x 128 x 64, four waves as 2 x 2, a wave owns WMT x 2 MFMA tiles of
-// 32 x 32.  WMT = 4 (256 x 128 blocks, 128 x 64 a wave) needs 6 operand fragments from LDS
-// for 8 MFMAs where WMT = 2 (128 x 128, 64 x 64 a wave) needs 4 for 4: LDS delivers 128
-// bytes a clock, one fragment per MFMA slot, so the larger wave tile is what lets the matrix
-// cores run ahead of LDS.  The smaller block is kept for shapes that would give too few blocks.
-#define GT_BN 128
+// Block tile (32 WMT NWM) x (64 NWN) x 64 with NWM x NWN waves; a wave owns WMT x 2 MFMA tiles
+// of 32 x 32.  The k tiles alternate between two LDS buffers: the loads of the next tile are
+// issued before the products of the current one and stored after them, one barrier a tile.
 #define GT_BK 64
 #define GT_LD (GT_BK + 8)
 
-template <int WMT, bool GATED>
-__global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict__ A, int lda,
-                                                        const __bf16* __restrict__ W,
-                                                        void* __restrict__ C, int ldc, int c_is_f32,
-                                                        int M, int N, int K, int epi, float cap,
-                                                        int tiles_m, int tiles_n, int w_strip) {
-  constexpr int BM = 64 * WMT;
-  constexpr int APT = BM / 32;                 // 16-byte pieces of A a thread moves per k tile
-  __shared__ __bf16 sA[BM][GT_LD];
-  __shared__ __bf16 sB[GT_BN][GT_LD];
+template <int WMT, int NWM, int NWN, bool GATED, bool EXACT>
+__global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_tile_kernel(
+    const __bf16* __restrict__ A, int lda, const __bf16* __restrict__ W, void* __restrict__ C, int ldc,
+    int c_is_f32, int M, int N, int K, int epi, float cap, int tiles_m, int tiles_n, int w_strip) {
+  constexpr int T = 64 * NWM * NWN;
+  constexpr int BM = 32 * WMT * NWM, BN = 64 * NWN;
+  constexpr int RPP = T / 8;                   // rows one pass of the block's threads covers
+  constexpr int APT = BM / RPP, BPT = BN / RPP;   // 16-byte pieces a thread moves per k tile
+  static_assert(BM % RPP == 0 && BN % RPP == 0 && (T / 64) % 2 == 0, "tile and thread counts do not fit");
+  extern __shared__ __align__(16) unsigned char gt_lds[];
+  typedef __bf16 (*tile_t)[GT_LD];
+  const tile_t tiles = (tile_t)gt_lds;          // buffer b: A rows, then W rows, from row b (BM + BN)
   // blocks that share a weight tile run on one XCD (ids go round-robin over 8 XCDs)
   int id = blockIdx.x;
   const int total = tiles_m * tiles_n;
   if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
   const int tn = id / tiles_m, tm = id % tiles_m;
   const int m0 = tm * BM;
-  const int ncols = GATED ? GT_BN / 2 : GT_BN;       // output columns of the block
-  const int n0 = tn * ncols;
+  constexpr int NCOLS = GATED ? BN / 2 : BN;         // output columns of the block
+  const int n0 = tn * NCOLS;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / NWN, wn = wave % NWN;
   const int lr = lane & 31, lk = lane >> 5;
 
-  // piece c = tid + 256 i of a tile: row c / 8, eight k values at (c % 8) * 8
+  // piece c = tid + T i of a tile: row c / 8, eight k values at (c % 8) * 8
   const int prow = tid >> 3, pcol = (tid & 7) * 8;
   const __bf16* ga[APT];
-  const __bf16* gb[4];
+  const __bf16* gb[BPT];
 #pragma unroll
-  for (int i = 0; i < APT; i++) ga[i] = A + (size_t)min(m0 + prow + 32 * i, M - 1) * lda + pcol;
-  int brow[4], bcol;      // where a thread's pieces of the weight tile land in LDS
+  for (int i = 0; i < APT; i++) ga[i] = A + (size_t)min(m0 + prow + RPP * i, M - 1) * lda;
+  int brow[BPT], bcol;      // where a thread's pieces of the weight tile land in LDS
   if (w_strip) {
-    // a wave copies whole KB blocks: block (tid / 64) + 4 i of the tile's 8 strips x 2 steps,
-    // lane l = tid % 64 its 16 bytes; the k tile advances by two steps = 1024 elements
-    const int l = tid & 63, tstep = (tid >> 6) & 1;
+    // a wave copies whole KB blocks: block wave + (T / 64) i of the tile's BN / 16 strips x 2
+    // steps, lane l its 16 bytes; the k tile advances by two steps = 1024 elements
+    const int tstep = wave & 1;
     const int ksteps = (K + 31) / 32;
     const int strips = GATED ? 2 * N / 16 : (N + 15) / 16;
-    bcol = tstep * 32 + (l >> 4) * 8;
+    bcol = tstep * 32 + (lane >> 4) * 8;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int sit = ((tid >> 6) + 4 * i) >> 1;            // strip within the tile
-      brow[i] = sit * 16 + (l & 15);
+    for (int i = 0; i < BPT; i++) {
+      const int sit = (wave + (T / 64) * i) >> 1;            // strip within the tile
+      brow[i] = sit * 16 + (lane & 15);
       int gs;
-      if (GATED) gs = sit < 4 ? n0 / 16 + sit : N / 16 + n0 / 16 + (sit - 4);
+      if (GATED) gs = sit < BN / 32 ? n0 / 16 + sit : N / 16 + n0 / 16 + (sit - BN / 32);
       else gs = n0 / 16 + sit;
       gs = min(gs, strips - 1);
-      gb[i] = W + ((size_t)gs * ksteps + tstep) * 512 + l * 8;
+      gb[i] = W + (size_t)gs * ksteps * 512 + lane * 8;
     }
   } else {
     bcol = pcol;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int row = prow + 32 * i;
+    for (int i = 0; i < BPT; i++) {
+      const int row = prow + RPP * i;
       brow[i] = row;
       int bn;
-      if (GATED) bn = row < 64 ? min(n0 + row, N - 1) : N + min(n0 + row - 64, N - 1);
+      if (GATED) bn = row < BN / 2 ? min(n0 + row, N - 1) : N + min(n0 + row - BN / 2, N - 1);
       else bn = min(n0 + row, N - 1);
-      gb[i] = W + (size_t)bn * K + pcol;
+      gb[i] = W + (size_t)bn * K;
     }
   }
-  const size_t bstep = w_strip ? 1024 : GT_BK;      // elements between a piece and the same piece one k tile on
+  // a piece's offset from its row's (strip's) first element: tile t, then the place in the tile
+  const int boff = w_strip ? (wave & 1) * 512 : pcol, bstep = w_strip ? 1024 : GT_BK;
   f32x16 acc[WMT][2];
 #pragma unroll
   for (int i = 0; i < WMT; i++)
@@ -227,38 +227,44 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-  bf16x8 ra[APT], rb[4];
-  {
-    const bool in = pcol < K, inb = bcol < K;
+  // Two register sets: the loads of tile t + 2 are issued while tile t is multiplied and tile
+  // t + 1 waits in the other set, so a load has a whole tile's products to arrive in.
+  bf16x8 ra0[APT], rb0[BPT], ra1[APT], rb1[BPT];
+  // EXACT (K a multiple of the k tile): no load is under a condition, so that the compiler
+  // can count the loads in flight and wait for the older set alone; a tile beyond K is read
+  // from the last tile instead and never multiplied.  Otherwise pieces beyond K are zeros.
+  auto fetch = [&](int k0, bf16x8 (&ra)[APT], bf16x8 (&rb)[BPT]) {
+    if (EXACT) {
+      const int kc = min(k0, K - GT_BK);
+      const int aoff = kc + pcol, woff = (kc / GT_BK) * bstep + boff;
 #pragma unroll
-    for (int i = 0; i < APT; i++) ra[i] = in ? *(const bf16x8*)(ga[i]) : zero8();
+      for (int i = 0; i < APT; i++) ra[i] = *(const bf16x8*)(ga[i] + aoff);
 #pragma unroll
-    for (int i = 0; i < 4; i++) rb[i] = inb ? *(const bf16x8*)(gb[i]) : zero8();
-  }
-  for (int k0 = 0; k0 < K; k0 += GT_BK) {
-    __syncthreads();
+      for (int i = 0; i < BPT; i++) rb[i] = *(const bf16x8*)(gb[i] + woff);
+    } else {
+      const bool in = k0 + pcol < K, inb = k0 + bcol < K;
 #pragma unroll
-    for (int i = 0; i < APT; i++) *(bf16x8*)(&sA[prow + 32 * i][pcol]) = ra[i];
+      for (int i = 0; i < APT; i++) ra[i] = in ? *(const bf16x8*)(ga[i] + k0 + pcol) : zero8();
 #pragma unroll
-    for (int i = 0; i < 4; i++) *(bf16x8*)(&sB[brow[i]][bcol]) = rb[i];
-    __syncthreads();
-    const int kn = k0 + GT_BK;
-    if (kn < K) {
-      const bool in = kn + pcol < K, inb = kn + bcol < K;
-#pragma unroll
-      for (int i = 0; i < APT; i++) ra[i] = in ? *(const bf16x8*)(ga[i] + kn) : zero8();
-#pragma unroll
-      for (int i = 0; i < 4; i++) rb[i] = inb ? *(const bf16x8*)(gb[i] + (size_t)(kn / GT_BK) * bstep) : zero8();
+      for (int i = 0; i < BPT; i++) rb[i] = inb ? *(const bf16x8*)(gb[i] + (k0 / GT_BK) * bstep + boff) : zero8();
     }
+  };
+  auto stash = [&](int buf, const bf16x8 (&ra)[APT], const bf16x8 (&rb)[BPT]) {
+#pragma unroll
+    for (int i = 0; i < APT; i++) *(bf16x8*)(&tiles[buf * (BM + BN) + prow + RPP * i][pcol]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < BPT; i++) *(bf16x8*)(&tiles[buf * (BM + BN) + BM + brow[i]][bcol]) = rb[i];
+  };
+  auto multiply = [&](int buf) {
 #pragma unroll
     for (int ks = 0; ks < GT_BK / 16; ks++) {
       bf16x8 fa[WMT], fb[2];
 #pragma unroll
-      for (int i = 0; i < WMT; i++) fa[i] = *(const bf16x8*)(&sA[wm * (32 * WMT) + i * 32 + lr][ks * 16 + lk * 8]);
+      for (int i = 0; i < WMT; i++) fa[i] = *(const bf16x8*)(&tiles[buf * (BM + BN) + wm * (32 * WMT) + i * 32 + lr][ks * 16 + lk * 8]);
 #pragma unroll
       for (int j = 0; j < 2; j++) {
-        const int brow = GATED ? j * 64 + wn * 32 : wn * 64 + j * 32;
-        fb[j] = *(const bf16x8*)(&sB[brow + lr][ks * 16 + lk * 8]);
+        const int row = GATED ? j * (BN / 2) + wn * 32 : wn * 64 + j * 32;
+        fb[j] = *(const bf16x8*)(&tiles[buf * (BM + BN) + BM + row + lr][ks * 16 + lk * 8]);
       }
 #pragma unroll
       for (int i = 0; i < WMT; i++)
@@ -266,6 +272,35 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
         for (int j = 0; j < 2; j++)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
     }
+  };
+  // The loop takes two tiles a turn.  An odd number of tiles: when EXACT the first tile is
+  // taken alone before the loop, otherwise the last one is all zeros.
+  int kfirst = 0;
+  if (EXACT && (K / GT_BK) % 2 == 1) {
+    fetch(0, ra0, rb0);
+    stash(0, ra0, rb0);
+    __syncthreads();
+    multiply(0);
+    __syncthreads();
+    kfirst = GT_BK;
+  }
+  if (kfirst < K) {
+    fetch(kfirst, ra0, rb0);
+    stash(0, ra0, rb0);
+    fetch(kfirst + GT_BK, ra0, rb0);
+    __syncthreads();
+  }
+  for (int k0 = kfirst; k0 < K; k0 += 2 * GT_BK) {
+    // tile k0 is in buffer 0, tile k0 + BK in set 0
+    fetch(k0 + 2 * GT_BK, ra1, rb1);
+    multiply(0);
+    stash(1, ra0, rb0);
+    __syncthreads();
+    // tile k0 + BK is in buffer 1, tile k0 + 2 BK in set 1
+    fetch(k0 + 3 * GT_BK, ra0, rb0);
+    multiply(1);
+    stash(0, ra1, rb1);
+    __syncthreads();
   }
   // acc[i][j][4*b + e] is row 8*b + 4*lk + e of the 32x32 tile, column lr
 #pragma unroll
@@ -299,6 +334,26 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const __bf16* __restrict
   }
 }
 
+template <int WMT, int NWM, int NWN, bool GATED, bool EXACT>
+static int launch_tile(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M, int N,
+                       int K, int epi, float cap, int w_strip, hipStream_t s) {
+  constexpr int BM = 32 * WMT * NWM, BN = 64 * NWN;
+  constexpr int ncols = GATED ? BN / 2 : BN;
+  constexpr size_t lds = (size_t)2 * (BM + BN) * GT_LD * sizeof(__bf16);
+  static bool prepared = false;
+  if (!prepared) {
+    if (lds > 64 * 1024 &&
+        hipFuncSetAttribute((const void*)gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return zk_fail("zk_gemm_bf16: the tile kernel's LDS buffers were refused");
+    prepared = true;
+  }
+  const int tiles_n = (N + ncols - 1) / ncols, tiles_m = (M + BM - 1) / BM;
+  ZK_REQUIRE((long long)tiles_m * tiles_n < 2147483647LL, "zk_gemm_bf16: too many tiles");
+  gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT><<<dim3(tiles_m * tiles_n), 64 * NWM * NWN, lds, s>>>(
+      (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, tiles_m, tiles_n, w_strip);
+  return zk_launch_status("zk_gemm_bf16 (tile)");
+}
 
 // ------------------------------------------------------------------ mid (16 < M <= 64)
 // With more than one column tile the activations weigh more than the weights on the way
@@ -561,22 +616,26 @@ extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int 
     return gated ? launch_skinny<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s)
                  : launch_skinny<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s);
   }
-  const int ncols = gated ? GT_BN / 2 : GT_BN;
-  const int tiles_n = (N + ncols - 1) / ncols;
-  // 128-row blocks (WMT = 2): three of them fit a CU and hide each other's waits.  The
-  // 256-row block (WMT = 4) halves LDS traffic per MFMA but runs one block a CU with its
-  // loads exposed; measured slower (608 vs 741 TFLOP/s at 2048 x 4096 x 2304) until the k loop
-  // is double-buffered, so it is not selected.
+  // 128 x 128 blocks of four waves (two share a CU) or 128 x 256 blocks of eight (one a CU,
+  // about 1.2 times the rate).  What counts is the CU with the most blocks; a lone small block
+  // runs at about 0.8 of the rate of two.  The constants are measured (M = 512 and 2048 with
+  // N = 2304 to 18432): the rule picked the faster of the two in each of those.
   const int tiles_m = (M + 127) / 128;
-  ZK_REQUIRE((long long)tiles_m * tiles_n < 2147483647LL, "zk_gemm_bf16: too many tiles");
-  dim3 grid(tiles_m * tiles_n);
-  if (gated)
-    gemm_tile_kernel<2, true><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32,
-                                                   M, N, K, epi, cap, tiles_m, tiles_n, w_strip);
-  else
-    gemm_tile_kernel<2, false><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32,
-                                                    M, N, K, epi, cap, tiles_m, tiles_n, w_strip);
-  return zk_launch_status("zk_gemm_bf16 (tile)");
+  const long nb_small = (long)tiles_m * ((N + (gated ? 64 : 128) - 1) / (gated ? 64 : 128));
+  const long nb_wide = (long)tiles_m * ((N + (gated ? 128 : 256) - 1) / (gated ? 128 : 256));
+  const long per_cu_small = (nb_small + 255) / 256, per_cu_wide = (nb_wide + 255) / 256;
+  const double cost_small = per_cu_small * 16384.0 / (per_cu_small == 1 ? 0.8 : 1.0);
+  const double cost_wide = per_cu_wide * 32768.0 / 1.2;
+  const bool wide = cost_wide < cost_small;
+  const bool exact = K % GT_BK == 0;
+#define ZK_TILE_(W_, M_, N_, G_, E_) launch_tile<W_, M_, N_, G_, E_>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s)
+#define ZK_TILE(W_, M_, N_)                                                                            \
+  (gated ? (exact ? ZK_TILE_(W_, M_, N_, true, true) : ZK_TILE_(W_, M_, N_, true, false))             \
+         : (exact ? ZK_TILE_(W_, M_, N_, false, true) : ZK_TILE_(W_, M_, N_, false, false)))
+  if (wide) return ZK_TILE(2, 2, 4);
+  return ZK_TILE(2, 2, 2);
+#undef ZK_TILE
+#undef ZK_TILE_
 }
 
 #endif  // ZSE_ACT_BF16
