@@ -62,12 +62,6 @@ struct AttnParams {
   int nchunks;            // split: chunks the grid covers
 };
 
-__device__ __forceinline__ float fast_tanh(float x) {
-  // tanh(x) = 1 - 2 / (exp(2x) + 1); exact at the ends, relative error ~1e-6 between
-  const float e = __expf(2.f * x);
-  return 1.f - 2.f / (e + 1.f);
-}
-
 __device__ __forceinline__ float score_log2(const AttnParams& p, float dot) {
   if (p.softcap > 0.f) {
     const float e = __builtin_amdgcn_exp2f(p.k2 * dot);

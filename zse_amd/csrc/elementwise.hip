@@ -180,13 +180,23 @@ __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
   const int r = blockIdx.x;
   const act_t* s = sub + (size_t)r * H;
   float* hr = h + (size_t)r * H;
-  float v[NF_MAXV][4];
+  // every load is issued before the first sum is needed: one trip to memory, not three
+  float v[NF_MAXV][4], hv[NF_MAXV][4], gp[NF_MAXV][4], gn[NF_MAXV][4];
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < NF_MAXV; j++) {
     const int i = threadIdx.x * 4 + j * 1024;
     if (i < H) {
       load4<act_t>(s + i, v[j]);
+      load4<float>(hr + i, hv[j]);
+      if (w_post) load4<float>(w_post + i, gp[j]);
+      if (w_next) load4<float>(w_next + i, gn[j]);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NF_MAXV; j++) {
+    const int i = threadIdx.x * 4 + j * 1024;
+    if (i < H) {
 #pragma unroll
       for (int e = 0; e < 4; e++) ss += v[j][e] * v[j][e];
     }
@@ -201,14 +211,11 @@ __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
   for (int j = 0; j < NF_MAXV; j++) {
     const int i = threadIdx.x * 4 + j * 1024;
     if (i < H) {
-      float g[4], hv[4];
-      load4<float>(hr + i, hv);
-      if (w_post) load4<float>(w_post + i, g);
 #pragma unroll
       for (int e = 0; e < 4; e++) {
         float t = v[j][e];
-        if (w_post) t = t * rs * (uo_post ? 1.f + g[e] : g[e]);
-        t = hv[e] + t;
+        if (w_post) t = t * rs * (uo_post ? 1.f + gp[j][e] : gp[j][e]);
+        t = hv[j][e] + t;
         v[j][e] = t;
         ss2 += t * t;
       }
@@ -223,10 +230,9 @@ __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
   for (int j = 0; j < NF_MAXV; j++) {
     const int i = threadIdx.x * 4 + j * 1024;
     if (i < H) {
-      float g[4], y[4];
-      load4<float>(w_next + i, g);
+      float y[4];
 #pragma unroll
-      for (int e = 0; e < 4; e++) y[e] = v[j][e] * rs2 * (uo_next ? 1.f + g[e] : g[e]);
+      for (int e = 0; e < 4; e++) y[e] = v[j][e] * rs2 * (uo_next ? 1.f + gn[j][e] : gn[j][e]);
       store4(o + i, y);
     }
   }
