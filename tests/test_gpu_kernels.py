@@ -57,7 +57,8 @@ def gelu(z):
 
 # ------------------------------------------------------------------ matrix products
 GEMM_SHAPES = [(1, 1000, 96), (7, 320, 320), (8, 2304, 2048), (16, 50, 64), (33, 1000, 328),
-               (64, 513, 1024), (65, 300, 96), (200, 1000, 320), (300, 257, 2304), (128, 128, 64)]
+               (64, 513, 1024), (65, 300, 96), (200, 1000, 320), (300, 257, 2304), (128, 128, 64),
+               (100, 200, 2048), (70, 90, 4168)]      # few tiles and a long K: split over blocks
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
@@ -85,6 +86,10 @@ def test_gemm_bf16_matrix_cores(rt, M, N, K):
     C = rt.empty((M, N), "float32")
     k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, N, 1, M, N, K, 0, 0.0, 0, None, 0, rt.stream)
     assert np.abs(rt.download(C) - want).max() < 1e-4 * math.sqrt(K)      # float accumulation
+    ws = gemm_workspace(rt)      # with a workspace a long K is split over blocks and joined
+    C2 = rt.empty((M, N), "float32")
+    k.zk_gemm_bf16(A.ptr, K, W.ptr, C2.ptr, N, 1, M, N, K, 0, 0.0, 0, ws.ptr, ws.nbytes, rt.stream)
+    assert np.abs(rt.download(C2) - want).max() < 1e-4 * math.sqrt(K)
     Cb = rt.empty((M, N), "bfloat16")
     k.zk_gemm_bf16(A.ptr, K, W.ptr, Cb.ptr, N, 0, M, N, K, 0, 0.0, 0, None, 0, rt.stream)
     got = rt.download_f32(Cb)
@@ -114,7 +119,10 @@ def test_gemm_bf16_gated_epilogue(rt, M, I, K, act):
                                           # 17..64 rows: activations shared in LDS, one to eight k chunks
                                           (17, 100, 64, False), (33, 2304, 2048, False), (48, 333, 544, False),
                                           (64, 1000, 512, False), (50, 72, 800, False), (20, 176, 288, True),
-                                          (64, 320, 800, True), (40, 336, 256, True), (33, 48, 1056, True)])
+                                          (64, 320, 800, True), (40, 336, 256, True), (33, 48, 1056, True),
+                                          # over 64 rows, few tiles, long K: k ranges over blocks, then a join
+                                          (100, 200, 2048, False), (130, 336, 2048, True), (70, 90, 4128, False),
+                                          (512, 2304, 9216, False)])
 def test_gemm_bf16_strip_layout(rt, M, N, K, gated):
     """The same products with the weights rearranged into strips of 16 rows by 32 columns, and
     an embedding gather out of that layout."""

@@ -157,10 +157,65 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
 #define GT_BK 64
 #define GT_LD (GT_BK + 8)
 
+// Blocks that share a weight tile run on one XCD (ids go round-robin over 8 XCDs).
+__device__ __forceinline__ void tile_of_block(int id, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
+  tn = id / tiles_m;
+  tm = id % tiles_m;
+}
+
+// Four results of a lane: rows 8 b + 4 lk + e (e = 0..3) of the wave's 32 x 32 tiles (i, 0) and
+// (i, 1), column lr; x0 belongs to tile (i, 0), x1 to tile (i, 1) (gate and up when GATED).
+template <int WMT, int NWN, bool GATED>
+__device__ __forceinline__ void tile_store_quad(const f32x4& x0, const f32x4& x1, int i, int b,
+                                                void* __restrict__ C, int ldc, int c_is_f32, int M, int N,
+                                                int m0, int n0, int wm, int wn, int lane, int epi, float cap) {
+  const int lr = lane & 31, lk = lane >> 5;
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    const int m = m0 + wm * (32 * WMT) + i * 32 + 8 * b + 4 * lk + e;
+    if (m >= M) continue;
+    if (GATED) {
+      const int n = n0 + wn * 32 + lr;
+      if (n < N) {
+        const float x = epi_gate(x0[e], x1[e], epi);
+        if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
+        else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const int n = n0 + wn * 64 + j * 32 + lr;
+        if (n >= N) continue;
+        float x = j ? x1[e] : x0[e];
+        if (epi == EPI_SOFTCAP) x = cap * tanhf(x / cap);
+        if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
+        else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
+      }
+    }
+  }
+}
+
+template <int WMT, int NWN, bool GATED>
+__device__ __forceinline__ void tile_store(const f32x16 (&acc)[WMT][2], void* __restrict__ C, int ldc,
+                                           int c_is_f32, int M, int N, int m0, int n0, int wm, int wn,
+                                           int lane, int epi, float cap) {
+#pragma unroll
+  for (int i = 0; i < WMT; i++)
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+      const f32x4 x0 = {acc[i][0][4 * b], acc[i][0][4 * b + 1], acc[i][0][4 * b + 2], acc[i][0][4 * b + 3]};
+      const f32x4 x1 = {acc[i][1][4 * b], acc[i][1][4 * b + 1], acc[i][1][4 * b + 2], acc[i][1][4 * b + 3]};
+      tile_store_quad<WMT, NWN, GATED>(x0, x1, i, b, C, ldc, c_is_f32, M, N, m0, n0, wm, wn, lane, epi, cap);
+    }
+}
+
 template <int WMT, int NWM, int NWN, bool GATED, bool EXACT>
 __global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_tile_kernel(
     const __bf16* __restrict__ A, int lda, const __bf16* __restrict__ W, void* __restrict__ C, int ldc,
-    int c_is_f32, int M, int N, int K, int epi, float cap, int tiles_m, int tiles_n, int w_strip) {
+    int c_is_f32, int M, int N, int K_all, int epi, float cap, int tiles_m, int tiles_n, int w_strip,
+    f32x16* __restrict__ partials, int ksplit) {
   constexpr int T = 64 * NWM * NWN;
   constexpr int BM = 32 * WMT * NWM, BN = 64 * NWN;
   constexpr int RPP = T / 8;                   // rows one pass of the block's threads covers
@@ -169,30 +224,33 @@ __global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_t
   extern __shared__ __align__(16) unsigned char gt_lds[];
   typedef __bf16 (*tile_t)[GT_LD];
   const tile_t tiles = (tile_t)gt_lds;          // buffer b: A rows, then W rows, from row b (BM + BN)
-  // blocks that share a weight tile run on one XCD (ids go round-robin over 8 XCDs)
-  int id = blockIdx.x;
-  const int total = tiles_m * tiles_n;
-  if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
-  const int tn = id / tiles_m, tm = id % tiles_m;
+  int tm, tn;
+  tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM;
   constexpr int NCOLS = GATED ? BN / 2 : BN;         // output columns of the block
   const int n0 = tn * NCOLS;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / NWN, wn = wave % NWN;
   const int lr = lane & 31, lk = lane >> 5;
+  // blockIdx.y takes a range of k tiles (the whole of K unless the launch splits it); the
+  // operand pointers start at the range, so below K counts from there
+  const int ktiles = (K_all + GT_BK - 1) / GT_BK;
+  const int kt0 = (int)((long)blockIdx.y * ktiles / ksplit), kt1 = (int)((long)(blockIdx.y + 1) * ktiles / ksplit);
+  const int kbase = kt0 * GT_BK;
+  const int K = min(K_all, kt1 * GT_BK) - kbase;
 
   // piece c = tid + T i of a tile: row c / 8, eight k values at (c % 8) * 8
   const int prow = tid >> 3, pcol = (tid & 7) * 8;
   const __bf16* ga[APT];
   const __bf16* gb[BPT];
 #pragma unroll
-  for (int i = 0; i < APT; i++) ga[i] = A + (size_t)min(m0 + prow + RPP * i, M - 1) * lda;
+  for (int i = 0; i < APT; i++) ga[i] = A + (size_t)min(m0 + prow + RPP * i, M - 1) * lda + kbase;
   int brow[BPT], bcol;      // where a thread's pieces of the weight tile land in LDS
   if (w_strip) {
     // a wave copies whole KB blocks: block wave + (T / 64) i of the tile's BN / 16 strips x 2
     // steps, lane l its 16 bytes; the k tile advances by two steps = 1024 elements
     const int tstep = wave & 1;
-    const int ksteps = (K + 31) / 32;
+    const int ksteps = (K_all + 31) / 32;
     const int strips = GATED ? 2 * N / 16 : (N + 15) / 16;
     bcol = tstep * 32 + (lane >> 4) * 8;
 #pragma unroll
@@ -203,7 +261,7 @@ __global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_t
       if (GATED) gs = sit < BN / 32 ? n0 / 16 + sit : N / 16 + n0 / 16 + (sit - BN / 32);
       else gs = n0 / 16 + sit;
       gs = min(gs, strips - 1);
-      gb[i] = W + (size_t)gs * ksteps * 512 + lane * 8;
+      gb[i] = W + ((size_t)gs * ksteps + 2 * kt0) * 512 + lane * 8;
     }
   } else {
     bcol = pcol;
@@ -214,7 +272,7 @@ __global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_t
       int bn;
       if (GATED) bn = row < BN / 2 ? min(n0 + row, N - 1) : N + min(n0 + row - BN / 2, N - 1);
       else bn = min(n0 + row, N - 1);
-      gb[i] = W + (size_t)bn * K;
+      gb[i] = W + (size_t)bn * K_all + kbase;
     }
   }
   // a piece's offset from its row's (strip's) first element: tile t, then the place in the tile
@@ -302,41 +360,49 @@ __global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_t
     stash(0, ra1, rb1);
     __syncthreads();
   }
-  // acc[i][j][4*b + e] is row 8*b + 4*lk + e of the 32x32 tile, column lr
+  if (ksplit > 1) {
+    // partial sums of this k range, in lane order; the join kernel adds the ranges up
+    f32x16* mine = partials + (((size_t)blockIdx.x * ksplit + blockIdx.y) * (NWM * NWN) + wave) * (WMT * 2 * 64) + lane;
 #pragma unroll
-  for (int i = 0; i < WMT; i++) {
+    for (int i = 0; i < WMT; i++)
 #pragma unroll
-    for (int b = 0; b < 4; b++) {
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const int m = m0 + wm * (32 * WMT) + i * 32 + 8 * b + 4 * lk + e;
-        if (m >= M) continue;
-        if (GATED) {
-          const int n = n0 + wn * 32 + lr;
-          if (n < N) {
-            const float x = epi_gate(acc[i][0][4 * b + e], acc[i][1][4 * b + e], epi);
-            if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
-            else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
-          }
-        } else {
-#pragma unroll
-          for (int j = 0; j < 2; j++) {
-            const int n = n0 + wn * 64 + j * 32 + lr;
-            if (n >= N) continue;
-            float x = acc[i][j][4 * b + e];
-            if (epi == EPI_SOFTCAP) x = cap * tanhf(x / cap);
-            if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
-            else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
-          }
-        }
-      }
-    }
+      for (int j = 0; j < 2; j++) mine[(i * 2 + j) * 64] = acc[i][j];
+    return;
   }
+  tile_store<WMT, NWN, GATED>(acc, C, ldc, c_is_f32, M, N, m0, n0, wm, wn, lane, epi, cap);
+}
+
+// Second half of a tile product whose K was split over blocks: the ranges are added in order.
+// A thread takes four consecutive floats of a lane's accumulator pair (i, 0), (i, 1), so the
+// partial sums are read in 16-byte pieces, neighbours by neighbouring threads.
+template <int WMT, int NWM, int NWN, bool GATED>
+__global__ __launch_bounds__(256) void gemm_tile_join_kernel(
+    const f32x4* __restrict__ partials, int ksplit, void* __restrict__ C, int ldc, int c_is_f32, int M,
+    int N, int epi, float cap, int tiles_m, int tiles_n) {
+  constexpr int BM = 32 * WMT * NWM, BN = 64 * NWN, NW = NWM * NWN;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const int b = (int)(idx & 3), lane = (int)((idx >> 2) & 63);
+  const int i = (int)((idx >> 8) % WMT), wave = (int)((idx >> 8) / WMT % NW);
+  const int tile = (int)((idx >> 8) / (WMT * NW));
+  if (tile >= tiles_m * tiles_n) return;
+  int tm, tn;
+  tile_of_block(tile, tiles_m, tiles_n, tm, tn);
+  // float4 index of (tile, range p, wave, pair member j, lane, b): an accumulator is 4 float4
+  const size_t per_wave = (size_t)WMT * 2 * 64 * 4;
+  const f32x4* src = partials + ((size_t)tile * ksplit * NW + wave) * per_wave + ((size_t)(i * 2) * 64 + lane) * 4 + b;
+  f32x4 x0 = src[0], x1 = src[64 * 4];
+  for (int p = 1; p < ksplit; p++) {
+    x0 += src[(size_t)p * NW * per_wave];
+    x1 += src[(size_t)p * NW * per_wave + 64 * 4];
+  }
+  tile_store_quad<WMT, NWN, GATED>(x0, x1, i, b, C, ldc, c_is_f32, M, N, tm * BM, tn * (GATED ? BN / 2 : BN),
+                                   wave / NWN, wave % NWN, lane, epi, cap);
 }
 
 template <int WMT, int NWM, int NWN, bool GATED, bool EXACT>
 static int launch_tile(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M, int N,
-                       int K, int epi, float cap, int w_strip, hipStream_t s) {
+                       int K, int epi, float cap, int w_strip, void* ws, size_t ws_bytes, int ksplit,
+                       hipStream_t s) {
   constexpr int BM = 32 * WMT * NWM, BN = 64 * NWN;
   constexpr int ncols = GATED ? BN / 2 : BN;
   constexpr size_t lds = (size_t)2 * (BM + BN) * GT_LD * sizeof(__bf16);
@@ -350,8 +416,16 @@ static int launch_tile(const void* A, int lda, const void* W, void* C, int ldc, 
   }
   const int tiles_n = (N + ncols - 1) / ncols, tiles_m = (M + BM - 1) / BM;
   ZK_REQUIRE((long long)tiles_m * tiles_n < 2147483647LL, "zk_gemm_bf16: too many tiles");
-  gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT><<<dim3(tiles_m * tiles_n), 64 * NWM * NWN, lds, s>>>(
-      (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, tiles_m, tiles_n, w_strip);
+  // K split over blockIdx.y only as far as the partial sums fit the workspace
+  const size_t per_range = (size_t)tiles_m * tiles_n * BM * BN * sizeof(float);
+  if (ws == nullptr || (uintptr_t)ws % 64 != 0) ksplit = 1;
+  while (ksplit > 1 && per_range * ksplit > ws_bytes) ksplit--;
+  gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT><<<dim3(tiles_m * tiles_n, ksplit), 64 * NWM * NWN, lds, s>>>(
+      (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, tiles_m, tiles_n, w_strip,
+      (f32x16*)ws, ksplit);
+  if (ksplit > 1)
+    gemm_tile_join_kernel<WMT, NWM, NWN, GATED><<<dim3(tiles_m * tiles_n * WMT * NWM * NWN), 256, 0, s>>>(
+        (const f32x4*)ws, ksplit, C, ldc, c_is_f32, M, N, epi, cap, tiles_m, tiles_n);
   return zk_launch_status("zk_gemm_bf16 (tile)");
 }
 
@@ -593,7 +667,7 @@ extern "C" int zk_strip_layout(const void* src, void* dst, int N, int K, void* s
 // gated epilogues, N % 16 == 0.
 // The workspace may be null; then K is never split over blocks.  It holds nothing between
 // launches and serves one launch at a time.
-extern "C" size_t zk_gemm_bf16_workspace() { return (size_t)16 << 20; }
+extern "C" size_t zk_gemm_bf16_workspace() { return (size_t)32 << 20; }
 
 extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
                             int M, int N, int K, int epi, float cap, int w_strip, void* ws,
@@ -628,7 +702,17 @@ extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int 
   const double cost_wide = per_cu_wide * 32768.0 / 1.2;
   const bool wide = cost_wide < cost_small;
   const bool exact = K % GT_BK == 0;
-#define ZK_TILE_(W_, M_, N_, G_, E_) launch_tile<W_, M_, N_, G_, E_>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s)
+  // Few small blocks: split K over blocks until about 320 blocks exist, a range no shorter than
+  // 8 k tiles, and the partial sums (4 M N bytes a range, written and read) no more than W.
+  int ksplit = 1;
+  if (!wide && nb_small < 160) {
+    ksplit = (int)(320 / nb_small);
+    ksplit = min(ksplit, (K + GT_BK - 1) / GT_BK / 8);
+    ksplit = min(ksplit, K / (4 * M));
+    ksplit = max(ksplit, 1);
+  }
+#define ZK_TILE_(W_, M_, N_, G_, E_) \
+  launch_tile<W_, M_, N_, G_, E_>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, ws, ws_bytes, ksplit, s)
 #define ZK_TILE(W_, M_, N_)                                                                            \
   (gated ? (exact ? ZK_TILE_(W_, M_, N_, true, true) : ZK_TILE_(W_, M_, N_, true, false))             \
          : (exact ? ZK_TILE_(W_, M_, N_, false, true) : ZK_TILE_(W_, M_, N_, false, false)))
