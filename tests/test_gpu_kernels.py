@@ -374,18 +374,25 @@ def test_gated_activation_and_softcap(rt, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("T", [27, 75])          # a block per (token, head); from 64 tokens a block per token
 @pytest.mark.parametrize("nh,nkv,hd,rot,bs,vt", [(4, 2, 16, 16, 4, 0), (6, 1, 32, 32, 8, 1), (8, 4, 256, 256, 16, 1),
                                                 (3, 3, 64, 32, 16, 0), (2, 2, 48, 0, 4, 1)])
-def test_rope_and_cache_write(rt, dtype, nh, nkv, hd, rot, bs, vt):
+def test_rope_and_cache_write(rt, dtype, T, nh, nkv, hd, rot, bs, vt):
     k = rt.kernels(dtype)
     rng = np.random.default_rng(hd)
-    T, pages = 7, 9
+    pages = 12
     qkv = rng.normal(size=(T, (nh + 2 * nkv) * hd)).astype(np.float32)
     if dtype == "bfloat16":
         qkv = bf16(qkv)
-    pos = np.array([0, 1, 5, 1000, 8191, 17, 3], np.int32)
-    slots = rng.permutation(pages * bs)[:T].astype(np.int32)
+    pos = np.concatenate([[0, 1, 5, 1000, 8191, 17, 3], rng.integers(0, 4000, T - 7)]).astype(np.int32)
+    slots = np.full(T, -1, np.int32)                         # tokens 27.. are not stored
+    slots[:27] = rng.permutation(9 * bs)[:27]                # scattered over pages 0..8
     slots[2] = -1                                            # nothing stored for this token
+    slots[8:16] = 9 * bs + np.arange(8) % bs                 # eight in a row from a page's start (if it has eight)
+    if bs < 8:
+        slots[12:16] = 10 * bs + np.arange(4) % bs
+    slots[16:24] = 11 * bs + (3 + np.arange(8)) % bs if bs >= 16 else slots[16:24]      # in a row, not aligned
+    assert len(set(slots[slots >= 0].tolist())) == (slots >= 0).sum()
     theta = 10000.0
     inv = (1.0 / theta ** (2.0 * np.arange(rot // 2) / max(rot, 1))).astype(np.float32)
     Q = up(rt, qkv, dtype)
