@@ -172,6 +172,9 @@ __global__ __launch_bounds__(256) void rmsnorm_fast_kernel(const TIn* __restrict
   }
 }
 
+// MAXV: vectors of four a thread holds (4 x 256 x MAXV >= H); small rows take fewer registers
+// and more rows share a CU.
+template <int MAXV>
 __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
     const act_t* __restrict__ sub, const float* __restrict__ w_post, float eps_post, int uo_post,
     float* __restrict__ h, const float* __restrict__ w_next, float eps_next, int uo_next,
@@ -181,10 +184,10 @@ __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
   const act_t* s = sub + (size_t)r * H;
   float* hr = h + (size_t)r * H;
   // every load is issued before the first sum is needed: one trip to memory, not three
-  float v[NF_MAXV][4], hv[NF_MAXV][4], gp[NF_MAXV][4], gn[NF_MAXV][4];
+  float v[MAXV][4], hv[MAXV][4], gp[MAXV][4], gn[MAXV][4];
   float ss = 0.f;
 #pragma unroll
-  for (int j = 0; j < NF_MAXV; j++) {
+  for (int j = 0; j < MAXV; j++) {
     const int i = threadIdx.x * 4 + j * 1024;
     if (i < H) {
       load4<act_t>(s + i, v[j]);
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
     }
   }
 #pragma unroll
-  for (int j = 0; j < NF_MAXV; j++) {
+  for (int j = 0; j < MAXV; j++) {
     const int i = threadIdx.x * 4 + j * 1024;
     if (i < H) {
 #pragma unroll
@@ -208,7 +211,7 @@ __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
   }
   float ss2 = 0.f;
 #pragma unroll
-  for (int j = 0; j < NF_MAXV; j++) {
+  for (int j = 0; j < MAXV; j++) {
     const int i = threadIdx.x * 4 + j * 1024;
     if (i < H) {
 #pragma unroll
@@ -227,7 +230,7 @@ __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
   const float rs2 = rsqrtf(ss2 / (float)H + eps_next);
   act_t* o = out + (size_t)r * H;
 #pragma unroll
-  for (int j = 0; j < NF_MAXV; j++) {
+  for (int j = 0; j < MAXV; j++) {
     const int i = threadIdx.x * 4 + j * 1024;
     if (i < H) {
       float y[4];
@@ -491,9 +494,13 @@ int zk_norm_add_norm(const void* sub, const float* w_post, float eps_post, int u
   ZK_REQUIRE(w_next == nullptr || out != nullptr, "zk_norm_add_norm: next norm without output");
   if (T == 0) return 0;
   if (H % 4 == 0 && H <= NF_MAXV * 1024) {
-    norm_add_norm_fast_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)sub, w_post, eps_post, uo_post,
-                                                                  h, w_next, eps_next, uo_next,
-                                                                  (act_t*)out, H);
+    if (H <= 3 * 1024)
+      norm_add_norm_fast_kernel<3><<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)sub, w_post, eps_post, uo_post,
+                                                                       h, w_next, eps_next, uo_next, (act_t*)out, H);
+    else
+      norm_add_norm_fast_kernel<NF_MAXV><<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)sub, w_post, eps_post,
+                                                                             uo_post, h, w_next, eps_next, uo_next,
+                                                                             (act_t*)out, H);
     return zk_launch_status("zk_norm_add_norm");
   }
   norm_add_norm_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)sub, w_post, eps_post, uo_post, h,
