@@ -217,6 +217,9 @@ ATT_CASES = [
     dict(nh=8, nkv=4, hd=256, bs=16, reqs=[(200, 45), (640, 1)], window=128, cap=0.0),
     dict(nh=32, nkv=16, hd=128, bs=32, reqs=[(5, 33), (255, 1), (256, 1)], window=100, cap=30.0),
     dict(nh=3, nkv=3, hd=64, bs=16, reqs=[(0, 2), (127, 1), (128, 2)], window=0, cap=0.0),
+    # many decoded tokens over long contexts: 64 keys a wave (fewer waves: 32)
+    dict(nh=8, nkv=4, hd=64, bs=16, reqs=[(1500, 1), (1499, 1), (1000, 1), (1343, 1), (1279, 1), (1280, 1)],
+         window=0, cap=50.0),
     dict(nh=10, nkv=2, hd=48, bs=16, reqs=[(3, 20), (60, 1)], window=24, cap=10.0),      # plain kernel only
 ]
 

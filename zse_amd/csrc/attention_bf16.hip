@@ -60,6 +60,7 @@ struct AttnParams {
   int tpw;                // tokens a wave owns
   int r_begin;            // first request of this launch
   int nchunks;            // split: chunks the grid covers
+  int chunk;              // decoded tokens on 16-wide tiles: keys a wave takes, 32 or 64
 };
 
 __device__ __forceinline__ float score_log2(const AttnParams& p, float dot) {
@@ -303,8 +304,8 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   if (n <= 0) return;
   const int pos = p.ctx_len[r] - 1;
   const int row_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
-  const int key_lo = max(row_lo, chunk * ATT_CHUNK);
-  const int key_hi = min(pos, chunk * ATT_CHUNK + ATT_CHUNK - 1);
+  const int key_lo = max(row_lo, chunk * p.chunk);
+  const int key_hi = min(pos, chunk * p.chunk + p.chunk - 1);
   const bool active = key_lo <= key_hi;          // a wave without keys still meets the others at the barrier
   const int g = p.nh / p.nkv;
   const bool col_ok = col < g;
@@ -418,7 +419,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   }
   __syncthreads();
   const int first_chunk = blockIdx.x * 4;
-  if (first_chunk * ATT_CHUNK > pos || first_chunk * ATT_CHUNK + 4 * ATT_CHUNK - 1 < row_lo) return;
+  if (first_chunk * p.chunk > pos || first_chunk * p.chunk + 4 * p.chunk - 1 < row_lo) return;
   for (int idx = threadIdx.x; idx < g * hd; idx += 256) {
     const int c = idx / hd, d = idx - c * hd;
     float mw[4], m = -INFINITY;
@@ -576,9 +577,16 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
     dim3 grid((nchunks + 3) / 4, nkv, n_dec);
     int rc = 0;
     int span = ATT_CHUNK;        // keys one partial result covers
+    p.chunk = ATT_CHUNK;
     if (g <= 16 && hd % 32 == 0) {
-      // the block joins its four chunks: one partial result per 4 * ATT_CHUNK keys
-      span = 4 * ATT_CHUNK;
+      // Few requests and a short context give few waves (one request at 4096 keys: 256 for
+      // 256 CUs), each a chain of two loads from memory; half the keys a wave then, one load.
+      if ((long long)n_dec * nkv * nchunks <= 512) {
+        p.chunk = ATT_CHUNK / 2;
+        grid.x = (2 * nchunks + 3) / 4;
+      }
+      // the block joins its four chunks: one partial result per 4 chunks of keys
+      span = 4 * p.chunk;
       p.nchunks = grid.x;
       p.part_ml = (float*)workspace + (size_t)n_dec * nh * p.nchunks * hd;
       const size_t lds = (4 * 16 * 2 + (size_t)4 * g * hd) * sizeof(float);
