@@ -160,6 +160,41 @@ def test_gemm_bf16_strip_layout(rt, M, N, K, gated):
         assert np.array_equal(rt.download(out), w[toks] * np.float32(2.0))
 
 
+def test_gemm_bf16_random_shapes(rt):
+    """Forty shapes drawn at random over the three kernels' ranges, both weight layouts, with
+    and without the gated epilogue and the workspace: whatever the dispatch picks must agree
+    with the product in float64."""
+    k = rt.kernels("bfloat16")
+    rng = np.random.default_rng(2024)
+    ws = gemm_workspace(rt)
+    for case in range(40):
+        M = int(rng.choice([rng.integers(1, 17), rng.integers(17, 65), rng.integers(65, 400)]))
+        strip = bool(rng.integers(0, 2))
+        gated = bool(rng.integers(0, 2))
+        K = int(rng.integers(1, 140)) * (32 if strip else 8)
+        N = int(rng.integers(1, 45)) * 16 if (gated and strip) else int(rng.integers(1, 700))
+        rows = 2 * N if gated else N
+        a, w = bf16(rng.normal(size=(M, K))), bf16(rng.normal(size=(rows, K)) * (0.3 if gated else 1.0))
+        A, W = up(rt, a, "bfloat16"), up(rt, w, "bfloat16")
+        if strip:
+            WS = rt.empty(((rows + 15) // 16 * 16, K), "bfloat16")
+            k.zk_strip_layout(W.ptr, WS.ptr, rows, K, rt.stream)
+            W = WS
+        C = rt.empty((M, N), "float32")
+        use_ws = bool(rng.integers(0, 2))
+        k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, N, 1, M, N, K, 2 if gated else 0, 0.0, 1 if strip else 0,
+                       ws.ptr if use_ws else None, ws.nbytes if use_ws else 0, rt.stream)
+        if gated:
+            g = a.astype(np.float64) @ w[:N].astype(np.float64).T
+            want = gelu(g) * (a.astype(np.float64) @ w[N:].astype(np.float64).T)
+            tol = 2e-4 * math.sqrt(K) * max(1.0, np.abs(want).max())
+        else:
+            want = a.astype(np.float64) @ w.astype(np.float64).T
+            tol = 1e-4 * math.sqrt(K)
+        err = np.abs(rt.download(C) - want).max()
+        assert err < tol, f"case {case}: M={M} N={N} K={K} strip={strip} gated={gated} workspace={use_ws}: {err}"
+
+
 def test_gemm_reference_vector(rt):
     # ones times 0.5 gives K * 0.5 (reference tests/test_modal_orchestrator.py:271-302)
     for dtype in ("float32", "bfloat16"):
