@@ -255,6 +255,8 @@ ATT_CASES = [
     # many decoded tokens over long contexts: 64 keys a wave (fewer waves: 32)
     dict(nh=8, nkv=4, hd=64, bs=16, reqs=[(1500, 1), (1499, 1), (1000, 1), (1343, 1), (1279, 1), (1280, 1)],
          window=0, cap=50.0),
+    # a portion whose row groups number 280: two groups a block (144 blocks run at once)
+    dict(nh=8, nkv=8, hd=16, bs=16, reqs=[(20, 1100)], window=300, cap=20.0),
     dict(nh=10, nkv=2, hd=48, bs=16, reqs=[(3, 20), (60, 1)], window=24, cap=10.0),      # plain kernel only
 ]
 

@@ -71,7 +71,7 @@ __device__ __forceinline__ float score_log2(const AttnParams& p, float dot) {
   return p.k1 * dot;
 }
 
-template <int HD16, bool SPLIT>
+template <int HD16, bool SPLIT, bool PAIR>
 __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
   constexpr int DT = (HD16 + 1) / 2;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -82,21 +82,26 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
   if (n <= 0) return;
   const int start = p.ctx_len[r] - n;
   // portions: a block owns one group of rows and its four waves take every fourth tile of
-  // keys (their results are joined at the end); decoded tokens: a wave owns one chunk of keys
-  const int gi = SPLIT ? 0 : blockIdx.x;
+  // keys (their results are joined at the end); or (PAIR) two neighbouring groups, waves 0
+  // and 2 the first, 1 and 3 the second, a group's two waves every second tile: half as many
+  // blocks, twice as long, for portions whose groups would need a second, half-empty round of
+  // blocks.  Decoded tokens: a wave owns one chunk of keys.
+  constexpr int WPG = PAIR ? 2 : 4;                             // waves a group
+  const int gi = SPLIT ? 0 : (PAIR ? blockIdx.x * 2 + (wave & 1) : blockIdx.x);
   const int chunk = SPLIT ? blockIdx.x * 4 + wave : 0;
   const int t0 = gi * p.tpw;
-  if (t0 >= n) return;
+  if ((SPLIT ? 0 : (PAIR ? blockIdx.x * 2 : blockIdx.x) * p.tpw) >= n) return;   // the whole block is past the portion
+  const bool group_ok = t0 < n;                                // else: no rows, the wave only meets the barriers
   const int g = p.nh / p.nkv;
   const int tok = lr / g, hq = lr - tok * g;
-  const int ntok = min(p.tpw, n - t0);
+  const int ntok = group_ok ? min(p.tpw, n - t0) : 0;
   const bool row_ok = tok < ntok;
   const int trow = qs + t0 + (row_ok ? tok : 0);
   const int pos = start + t0 + (row_ok ? tok : 0);
   const int head = kvh * g + (row_ok ? hq : 0);
   const int pos_lo = start + t0, pos_hi = start + t0 + ntok - 1;
   int key_lo = p.window > 0 ? max(0, pos_lo - p.window + 1) : 0;
-  int key_hi = pos_hi;
+  int key_hi = group_ok ? pos_hi : -1;
   if (SPLIT) {
     key_lo = max(key_lo, chunk * ATT_CHUNK);
     key_hi = min(key_hi, chunk * ATT_CHUNK + ATT_CHUNK - 1);
@@ -124,7 +129,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
     for (int e = 0; e < 16; e++) o[dt][e] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  for (int key0 = (key_lo / 32) * 32 + (SPLIT ? 0 : wave * 32); key0 <= key_hi; key0 += SPLIT ? 32 : 128) {
+  for (int key0 = (key_lo / 32) * 32 + (SPLIT ? 0 : (PAIR ? wave >> 1 : wave) * 32); key0 <= key_hi;
+       key0 += SPLIT ? 32 : 32 * WPG) {
     // ---- S^T = K Q^T
     f32x16 s;
 #pragma unroll
@@ -219,8 +225,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
         if (d < hd) *(f32x4*)(po + d) = f32x4{o[dt][4 * j], o[dt][4 * j + 1], o[dt][4 * j + 2], o[dt][4 * j + 3]};
       }
   } else {
-    // join the four waves' partial results: common maximum and sum per row, then the
-    // accumulators meet in LDS (waves 2, 3 -> 0, 1; then 1 -> 0)
+    // join a group's waves: common maximum and sum per row, then the accumulators meet in
+    // LDS (waves 2, 3 -> 0, 1; with four waves a group then 1 -> 0)
     extern __shared__ float dyn[];
     float* sm_ml = dyn;                          // [4][32][2]
     float* sm_o = dyn + 4 * 32 * 2;              // [2][DT * 16][64]
@@ -231,10 +237,10 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
     __syncthreads();
     float m_all = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 4; w++) m_all = fmaxf(m_all, sm_ml[(w * 32 + lr) * 2]);
+    for (int w = PAIR ? wave & 1 : 0; w < 4; w += PAIR ? 2 : 1) m_all = fmaxf(m_all, sm_ml[(w * 32 + lr) * 2]);
     float l_all = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; w++) {
+    for (int w = PAIR ? wave & 1 : 0; w < 4; w += PAIR ? 2 : 1) {
       const float mw = sm_ml[(w * 32 + lr) * 2];
       l_all += mw == -INFINITY ? 0.f : sm_ml[(w * 32 + lr) * 2 + 1] * __builtin_amdgcn_exp2f(mw - m_all);
     }
@@ -258,19 +264,23 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
 #pragma unroll
         for (int e = 0; e < 16; e++) o[dt][e] += src[(dt * 16 + e) * 64 + lane];
     }
-    __syncthreads();
-    if (wave == 1) {
+    if (!PAIR) {
+      __syncthreads();
+      if (wave == 1) {
 #pragma unroll
-      for (int dt = 0; dt < DT; dt++)
+        for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-        for (int e = 0; e < 16; e++) sm_o[(dt * 16 + e) * 64 + lane] = o[dt][e];
+          for (int e = 0; e < 16; e++) sm_o[(dt * 16 + e) * 64 + lane] = o[dt][e];
+      }
+      __syncthreads();
+      if (wave == 0) {
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+          for (int e = 0; e < 16; e++) o[dt][e] += sm_o[(dt * 16 + e) * 64 + lane];
+      }
     }
-    __syncthreads();
-    if (wave != 0 || !row_ok) return;
-#pragma unroll
-    for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-      for (int e = 0; e < 16; e++) o[dt][e] += sm_o[(dt * 16 + e) * 64 + lane];
+    if (wave >= (PAIR ? 2 : 1) || !row_ok) return;
     const float inv = 1.f / l_all;
     __bf16* orow = p.out + ((size_t)trow * p.nh + head) * hd;
 #pragma unroll
@@ -497,16 +507,16 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
   }
 }
 
-template <bool SPLIT>
+template <bool SPLIT, bool PAIR>
 static int launch_attn(const AttnParams& p, dim3 grid, hipStream_t s) {
   // the join of a portion's four waves needs [4][32][2] + [2][ceil(hd/32) * 16][64] floats of LDS
   const size_t lds = SPLIT ? 0 : (4 * 32 * 2 + (size_t)2 * ((p.hd + 31) / 32) * 16 * 64) * sizeof(float);
   switch (p.hd / 16) {
-    case 1: attn_mfma_kernel<1, SPLIT><<<grid, 256, lds, s>>>(p); break;
-    case 2: attn_mfma_kernel<2, SPLIT><<<grid, 256, lds, s>>>(p); break;
-    case 4: attn_mfma_kernel<4, SPLIT><<<grid, 256, lds, s>>>(p); break;
-    case 8: attn_mfma_kernel<8, SPLIT><<<grid, 256, lds, s>>>(p); break;
-    case 16: attn_mfma_kernel<16, SPLIT><<<grid, 256, lds, s>>>(p); break;
+    case 1: attn_mfma_kernel<1, SPLIT, PAIR><<<grid, 256, lds, s>>>(p); break;
+    case 2: attn_mfma_kernel<2, SPLIT, PAIR><<<grid, 256, lds, s>>>(p); break;
+    case 4: attn_mfma_kernel<4, SPLIT, PAIR><<<grid, 256, lds, s>>>(p); break;
+    case 8: attn_mfma_kernel<8, SPLIT, PAIR><<<grid, 256, lds, s>>>(p); break;
+    case 16: attn_mfma_kernel<16, SPLIT, PAIR><<<grid, 256, lds, s>>>(p); break;
     default: return zk_fail("zk_attention_bf16: head_dim must be 16, 32, 64, 128 or 256");
   }
   return zk_launch_status("zk_attention_bf16");
@@ -561,8 +571,12 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
     ZK_REQUIRE(max_q_len > 0, "zk_attention_bf16: max_q_len must be positive");
     p.tpw = 32 / g; p.r_begin = 0; p.nchunks = 1; p.part_o = nullptr; p.part_ml = nullptr;
     const int groups = (max_q_len + p.tpw - 1) / p.tpw;
-    dim3 grid(groups, nkv, r_prefill);
-    int rc = launch_attn<false>(p, grid, s);
+    // one block a group; two groups a block when that lets every block run at once (256 CUs,
+    // one block each) where single groups would need a second round
+    const long long single = (long long)groups * nkv * r_prefill, paired = (long long)((groups + 1) / 2) * nkv * r_prefill;
+    int rc;
+    if (single > 256 && paired <= 256) rc = launch_attn<false, true>(p, dim3((groups + 1) / 2, nkv, r_prefill), s);
+    else rc = launch_attn<false, false>(p, dim3(groups, nkv, r_prefill), s);
     if (rc) return rc;
   }
   const int n_dec = R - r_prefill;
@@ -598,7 +612,7 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
       }
       rc = zk_launch_status("zk_attention_bf16 (decode)");
     } else {
-      rc = launch_attn<true>(p, grid, s);
+      rc = launch_attn<true, false>(p, grid, s);
     }
     if (rc) return rc;
     ZK_REQUIRE(nchunks <= ATT_MAX_CHUNKS, "zk_attention_bf16: context too long for the split variant");
