@@ -82,26 +82,47 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
   if (n <= 0) return;
   const int start = p.ctx_len[r] - n;
   // portions: a block owns one group of rows and its four waves take every fourth tile of
-  // keys (their results are joined at the end); or (PAIR) two neighbouring groups, waves 0
-  // and 2 the first, 1 and 3 the second, a group's two waves every second tile: half as many
-  // blocks, twice as long, for portions whose groups would need a second, half-empty round of
-  // blocks.  Decoded tokens: a wave owns one chunk of keys.
-  constexpr int WPG = PAIR ? 2 : 4;                             // waves a group
-  const int gi = SPLIT ? 0 : (PAIR ? blockIdx.x * 2 + (wave & 1) : blockIdx.x);
+  // keys (their results are joined at the end).  Or (PAIR, for portions whose groups would
+  // need a second, half-empty round of blocks) two groups: one from the end of the portion,
+  // which sees many keys, and its mirror from the start, which sees few, so that every block
+  // has about the same work; the four waves are shared out between the two by their numbers
+  // of key tiles (3 + 1, 2 + 2 or 1 + 3), a group's waves taking its tiles in turn.
+  // Decoded tokens: a wave owns one chunk of keys.
+  int gi = 0, phase = wave, nphase = 4, first_wave = 0;        // group, and the wave's place among its waves
+  int na_block = 4;                                            // waves of the block's first group
+  if (!SPLIT && !PAIR) gi = blockIdx.x;
+  if (PAIR) {
+    const int groups = (n + p.tpw - 1) / p.tpw;
+    if ((int)blockIdx.x >= (groups + 1) / 2) return;           // the whole block is past the portion
+    const int ga = groups - 1 - blockIdx.x, gb = blockIdx.x;
+    if (ga != gb) {
+      auto tiles_of = [&](int gr) {
+        const int lo = start + gr * p.tpw, hi = start + min(n, (gr + 1) * p.tpw) - 1;
+        const int klo = p.window > 0 ? max(0, lo - p.window + 1) : 0;
+        return hi / 32 - klo / 32 + 1;
+      };
+      const int ta = tiles_of(ga), tb = tiles_of(gb);
+      const int na = min(3, max(1, (4 * ta + (ta + tb) / 2) / (ta + tb)));
+      na_block = na;
+      if (wave < na) { gi = ga; phase = wave; nphase = na; }
+      else { gi = gb; phase = wave - na; nphase = 4 - na; first_wave = na; }
+    } else {
+      gi = ga;
+    }
+  }
   const int chunk = SPLIT ? blockIdx.x * 4 + wave : 0;
   const int t0 = gi * p.tpw;
-  if ((SPLIT ? 0 : (PAIR ? blockIdx.x * 2 : blockIdx.x) * p.tpw) >= n) return;   // the whole block is past the portion
-  const bool group_ok = t0 < n;                                // else: no rows, the wave only meets the barriers
+  if (!PAIR && t0 >= n) return;
   const int g = p.nh / p.nkv;
   const int tok = lr / g, hq = lr - tok * g;
-  const int ntok = group_ok ? min(p.tpw, n - t0) : 0;
+  const int ntok = min(p.tpw, n - t0);
   const bool row_ok = tok < ntok;
   const int trow = qs + t0 + (row_ok ? tok : 0);
   const int pos = start + t0 + (row_ok ? tok : 0);
   const int head = kvh * g + (row_ok ? hq : 0);
   const int pos_lo = start + t0, pos_hi = start + t0 + ntok - 1;
   int key_lo = p.window > 0 ? max(0, pos_lo - p.window + 1) : 0;
-  int key_hi = group_ok ? pos_hi : -1;
+  int key_hi = pos_hi;
   if (SPLIT) {
     key_lo = max(key_lo, chunk * ATT_CHUNK);
     key_hi = min(key_hi, chunk * ATT_CHUNK + ATT_CHUNK - 1);
@@ -129,8 +150,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
     for (int e = 0; e < 16; e++) o[dt][e] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  for (int key0 = (key_lo / 32) * 32 + (SPLIT ? 0 : (PAIR ? wave >> 1 : wave) * 32); key0 <= key_hi;
-       key0 += SPLIT ? 32 : 32 * WPG) {
+  for (int key0 = (key_lo / 32) * 32 + (SPLIT ? 0 : phase * 32); key0 <= key_hi; key0 += SPLIT ? 32 : 32 * nphase) {
     // ---- S^T = K Q^T
     f32x16 s;
 #pragma unroll
@@ -225,8 +245,8 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
         if (d < hd) *(f32x4*)(po + d) = f32x4{o[dt][4 * j], o[dt][4 * j + 1], o[dt][4 * j + 2], o[dt][4 * j + 3]};
       }
   } else {
-    // join a group's waves: common maximum and sum per row, then the accumulators meet in
-    // LDS (waves 2, 3 -> 0, 1; with four waves a group then 1 -> 0)
+    // join a group's waves: common maximum and sum per row, then the accumulators of the
+    // group's other waves reach its first wave through LDS, one wave a round (a slot a group)
     extern __shared__ float dyn[];
     float* sm_ml = dyn;                          // [4][32][2]
     float* sm_o = dyn + 4 * 32 * 2;              // [2][DT * 16][64]
@@ -236,11 +256,9 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
     }
     __syncthreads();
     float m_all = -INFINITY;
-#pragma unroll
-    for (int w = PAIR ? wave & 1 : 0; w < 4; w += PAIR ? 2 : 1) m_all = fmaxf(m_all, sm_ml[(w * 32 + lr) * 2]);
+    for (int w = first_wave; w < first_wave + nphase; w++) m_all = fmaxf(m_all, sm_ml[(w * 32 + lr) * 2]);
     float l_all = 0.f;
-#pragma unroll
-    for (int w = PAIR ? wave & 1 : 0; w < 4; w += PAIR ? 2 : 1) {
+    for (int w = first_wave; w < first_wave + nphase; w++) {
       const float mw = sm_ml[(w * 32 + lr) * 2];
       l_all += mw == -INFINITY ? 0.f : sm_ml[(w * 32 + lr) * 2 + 1] * __builtin_amdgcn_exp2f(mw - m_all);
     }
@@ -249,38 +267,25 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
     for (int dt = 0; dt < DT; dt++)
 #pragma unroll
       for (int e = 0; e < 16; e++) o[dt][e] *= f;
-    if (wave >= 2) {
-      float* dst = sm_o + (size_t)(wave - 2) * DT * 16 * 64;
-#pragma unroll
-      for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-        for (int e = 0; e < 16; e++) dst[(dt * 16 + e) * 64 + lane] = o[dt][e];
-    }
-    __syncthreads();
-    if (wave < 2) {
-      const float* src = sm_o + (size_t)wave * DT * 16 * 64;
-#pragma unroll
-      for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-        for (int e = 0; e < 16; e++) o[dt][e] += src[(dt * 16 + e) * 64 + lane];
-    }
-    if (!PAIR) {
-      __syncthreads();
-      if (wave == 1) {
+    float* slot = sm_o + (size_t)(first_wave ? 1 : 0) * DT * 16 * 64;
+    const int rounds = max(na_block, 4 - na_block) - 1;
+    for (int step = 1; step <= rounds; step++) {
+      if (phase == step) {
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-          for (int e = 0; e < 16; e++) sm_o[(dt * 16 + e) * 64 + lane] = o[dt][e];
+          for (int e = 0; e < 16; e++) slot[(dt * 16 + e) * 64 + lane] = o[dt][e];
       }
       __syncthreads();
-      if (wave == 0) {
+      if (phase == 0 && step < nphase) {
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-          for (int e = 0; e < 16; e++) o[dt][e] += sm_o[(dt * 16 + e) * 64 + lane];
+          for (int e = 0; e < 16; e++) o[dt][e] += slot[(dt * 16 + e) * 64 + lane];
       }
+      __syncthreads();
     }
-    if (wave >= (PAIR ? 2 : 1) || !row_ok) return;
+    if (phase != 0 || !row_ok) return;
     const float inv = 1.f / l_all;
     __bf16* orow = p.out + ((size_t)trow * p.nh + head) * hd;
 #pragma unroll
