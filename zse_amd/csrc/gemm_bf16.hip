@@ -495,12 +495,18 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) acc[g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // Every load is issued, none under a condition (loads under a branch make the compiler wait
+  // for all loads in flight before the first use of any): a step past the range reads the
+  // range's last step again, a row past M row M - 1, and the activations are set to zero
+  // afterwards where they lie outside, which makes the product nothing whatever the weights.
   auto fetch_a = [&](int s0, bf16x8 (&ra)[APT]) {
 #pragma unroll
     for (int j = 0; j < APT; j++) {
       const int row = a_row0 + 8 * j;
-      const int k = s0 * 32 + a_piece * 8;
-      ra[j] = (row < M && s0 + a_piece / 4 < s_end) ? *(const bf16x8*)(A + (size_t)row * lda + k) : zero8();
+      const bool in = row < M && s0 + a_piece / 4 < s_end;
+      const int step = min(s0 + a_piece / 4, s_end - 1);
+      const bf16x8 v = *(const bf16x8*)(A + (size_t)min(row, M - 1) * lda + step * 32 + (a_piece % 4) * 8);
+      ra[j] = in ? v : zero8();
     }
   };
   auto stash_a = [&](int buf, const bf16x8 (&ra)[APT]) {
@@ -512,7 +518,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
     for (int s = 0; s < GM_STEPS; s++)
 #pragma unroll
       for (int g = 0; g < NS; g++)
-        wf[g][s] = (strip_ok && s0 + s < s_end) ? *(const bf16x8*)(wp[g] + (size_t)(s0 + s) * 512) : zero8();
+        wf[g][s] = *(const bf16x8*)(wp[g] + (size_t)min(s0 + s, s_end - 1) * 512);
   };
   auto multiply = [&](int buf, const bf16x8 (&wf)[NS][GM_STEPS]) {
 #pragma unroll
