@@ -27,6 +27,14 @@ GEMMA2_2B = dict(
     max_position_embeddings=8192)
 
 
+# further sizes of the same architecture, for looking beyond the default (--model)
+GEMMA2_9B = dict(GEMMA2_2B, num_hidden_layers=42, hidden_size=3584, num_attention_heads=16, num_key_value_heads=8,
+                 head_dim=256, query_pre_attn_scalar=256, intermediate_size=14336)
+GEMMA2_27B = dict(GEMMA2_2B, num_hidden_layers=46, hidden_size=4608, num_attention_heads=32, num_key_value_heads=16,
+                  head_dim=128, query_pre_attn_scalar=144, intermediate_size=36864)
+MODELS = {"2b": GEMMA2_2B, "9b": GEMMA2_9B, "27b": GEMMA2_27B}
+
+
 def weight_bytes(cfg, item=2):
     H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     nh, nkv, hd, L = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["num_hidden_layers"]
@@ -68,6 +76,7 @@ def main():
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated")
+    ap.add_argument("--model", choices=sorted(MODELS), default="2b", help="layer sizes: Gemma 2 2B (the default), 9B or 27B")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="profiling aid: run one of the two workloads (the JSON line then lacks the other)")
@@ -81,7 +90,7 @@ def main():
     from zse_amd.runtime.device import Runtime
     from zse_amd.sampling.sampler import DeviceSampler, SamplingParams
 
-    cfg = dict(GEMMA2_2B)
+    cfg = dict(MODELS[a.model])
     full_layers = cfg["num_hidden_layers"]
     if a.layers:
         cfg["num_hidden_layers"] = a.layers
@@ -166,11 +175,11 @@ def main():
 
     tok_s, step_s, byts = results[a.batch]
     out = {
-        "metric": "decode tok/s, Gemma 2 2B bf16, batch %d" % a.batch,
+        "metric": "decode tok/s, Gemma 2 %s bf16, batch %d" % (a.model.upper(), a.batch),
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"model": "gemma2-2b-shapes-random", "layers": cfg["num_hidden_layers"],
+        "config": {"model": f"gemma2-{a.model}-shapes-random", "layers": cfg["num_hidden_layers"],
                    "layers_full": full_layers, "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
                    "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
