@@ -144,13 +144,26 @@ def main():
                 n = min(left, T)
                 runner.step([StepEntry(r, rng.integers(0, V, n).tolist(), [])], download=False)
                 left -= n
-        last = rng.integers(0, V, B).tolist()
+        first = rng.integers(0, V, B).tolist()
         rows = [{"params": greedy, "u": 0.0} for _ in range(B)]
+        # As the engine decodes: the sampling kernel leaves the ids on the device, the next step
+        # takes them from there, and the host reads them four steps at a time (it has to, for
+        # stop tokens) while the next steps are already enqueued.
+        sampler.prepare_run(rows, [[0.0] * B])
+        pending, fed = [], None
 
         def one():
-            nonlocal last
-            logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(reqs, last)], download=False)
-            last = sampler.sample(logits, rows)
+            nonlocal fed
+            toks = first if fed is None else [0] * B
+            logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(reqs, toks)], download=False,
+                                 tokens_from=fed)
+            ids = sampler.sample_deferred(logits, 0)
+            fed = ids.device_ptr
+            pending.append(ids)
+            if len(pending) == 4:
+                for p in pending:
+                    p.result()
+                pending.clear()
         for _ in range(warmup):
             one()
         rt.sync()

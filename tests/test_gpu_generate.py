@@ -67,6 +67,49 @@ def test_greedy_generation_bfloat16(tiny_folders):
             toks.append(t)
 
 
+@pytest.mark.parametrize("temperature", [0.0, 0.9])
+def test_runs_of_steps_without_the_host_give_the_same_tokens(tiny_folders, temperature):
+    """Decoding several steps in a row before the host reads an id (the ids go from step to step
+    on the device) gives what step-by-step decoding gives: same tokens, same ends by length and
+    by stop token (found late: the output is cut back to it), also when pages run short in the
+    middle of a run and a request has to be recomputed."""
+    from zse_amd.engine.engine import Engine
+    from zse_amd.engine.request import FinishReason
+    from zse_amd.sampling import SamplingParams
+    cfg = TINY["B"][0]
+    folder = tiny_folders[("B", "float32")]
+    prompts = [random_tokens(cfg["vocab_size"], n, 70 + n) for n in (3, 9, 14, 6)]
+
+    def run(decode_run, num_blocks, stops):
+        eng = Engine(folder, dtype="float32", block_size=8, num_blocks=num_blocks, max_batch_tokens=32,
+                     max_batch_seqs=4, prefill_chunk_size=7, max_seq_len=128, decode_run=decode_run)
+        reqs = [eng.add_request(p, SamplingParams(max_tokens=m, temperature=temperature, seed=11 + i,
+                                                  stop_tokens=stops))
+                for i, (p, m) in enumerate(zip(prompts, (21, 5, 30, 13)))]
+        eng.run()
+        out = [(list(r.output_tokens), r.finish_reason) for r in reqs]
+        st = eng.stats()
+        assert st.generated_tokens == sum(len(o) for o, _ in out)
+        assert all(pool.free_pages == pool.num_pages for pool in eng.runner.manager.pools)
+        eng.close()
+        return out, st
+
+    base, _ = run(1, 64, ())
+    assert all(-1 not in o for o, _ in base)
+    got, st = run(4, 64, ())
+    assert got == base and st.steps >= 30
+    # a stop token that some request produces in the middle of its output
+    stop = base[2][0][len(base[2][0]) // 2]
+    want, _ = run(1, 64, (stop,))
+    assert any(r == FinishReason.STOP for _, r in want)
+    assert run(4, 64, (stop,))[0] == want
+    assert run(7, 64, (stop,))[0] == want
+    # so few pages that a request is preempted and computed again while others are in a run
+    tight, st1 = run(1, 8, ())
+    assert st1.preemptions > 0 and [o for o, _ in tight] == [o for o, _ in base]
+    assert run(4, 8, ())[0] == tight
+
+
 def test_sampled_requests_do_not_depend_on_the_batch(tiny_folders):
     """Temperature 0.8 with seed 7: the same tokens alone, in a batch, under another chunk size
     and after a forced recomputation; each token is what the plain sampler draws from the

@@ -41,7 +41,7 @@ class Engine:
                  num_blocks: Optional[int] = None, max_batch_tokens: int = 4096,
                  max_batch_seqs: int = 64, prefill_chunk_size: int = 512,
                  max_seq_len: Optional[int] = None, device_index: int = 0, tuned: bool = True,
-                 use_graphs: bool = True, quiet: bool = True):
+                 use_graphs: bool = True, quiet: bool = True, decode_run: int = 4):
         self.rt = Runtime.get(device_index)
         self.dtype = canonical_dtype(dtype)
         self.model = load_model(model, self.dtype, self.rt, tuned=tuned) if isinstance(model, str) else model
@@ -65,6 +65,11 @@ class Engine:
         self._stats = EngineStats()
         self._next_id = 0
         self.quiet = quiet
+        # Steps of single tokens in a row that are enqueued before the host looks at the ids
+        # they produced (1: look after every step).  The ids are fed from step to step on the
+        # device; a stop token found afterwards cuts the request's output back to it.
+        self.decode_run = max(1, int(decode_run))
+        self._next_plan: Optional[StepPlan] = None
 
     # ---- requests
     def add_request(self, prompt_tokens: Sequence[int], params: Optional[SamplingParams] = None,
@@ -85,9 +90,12 @@ class Engine:
 
     def step(self) -> List[Request]:
         """Schedule, run and sample one step; returns the requests that finished in it."""
-        plan = self.scheduler.schedule()
+        plan, self._next_plan = self._next_plan or self.scheduler.schedule(), None
         if not plan:
             return list(plan.failed)
+        run = self._run_length(plan)
+        if run >= 2:
+            return self._decode_run(plan, run)
         entries = [StepEntry(s.request.request_id,
                              s.request.all_tokens[s.start:s.start + s.count],
                              [s.count - 1] if s.sample else []) for s in plan.items]
@@ -106,6 +114,69 @@ class Engine:
         self._stats.generated_tokens += len(ids)
         self._stats.preemptions = self.scheduler.num_preemptions
         return done + list(plan.failed)
+
+    # ---- several steps of single tokens without waiting for the host in between
+    def _rows(self, plan: StepPlan, ahead: int = 0) -> List[dict]:
+        return [{"params": s.request.params, "u": uniform(s.request.seed, len(s.request.output_tokens) + ahead),
+                 "past": ()} for s in plan.items if s.sample]
+
+    def _run_length(self, plan: StepPlan) -> int:
+        """How many steps can follow each other before the host reads an id: every request
+        decodes, is sampled on the device in one manner, nobody waits to be admitted, and
+        nobody reaches its length before the run's last step."""
+        if self.decode_run < 2 or self.scheduler.waiting or plan.preempted or plan.failed:
+            return 1
+        if not all(s.count == 1 and s.sample and s.request.state == RequestState.DECODING for s in plan.items):
+            return 1
+        if not self.sampler.can_defer(self._rows(plan)):
+            return 1
+        n = self.decode_run
+        for s in plan.items:
+            r = s.request
+            n = min(n, r.params.max_tokens - len(r.output_tokens), self.runner.manager.max_model_len - r.num_tokens)
+        return n
+
+    def _decode_run(self, plan: StepPlan, length: int) -> List[Request]:
+        sch, runner, sampler = self.scheduler, self.runner, self.sampler
+        reqs = [s.request for s in plan.items]
+        first_len = [len(r.output_tokens) for r in reqs]
+        sampler.prepare_run(self._rows(plan), [[uniform(r.seed, n0 + i) for r, n0 in zip(reqs, first_len)]
+                                               for i in range(length)])
+        pending, done, tokens_from = [], [], None
+        for i in range(length):
+            known = tokens_from is None
+            entries = [StepEntry(r.request_id, [r.all_tokens[s.start] if known else 0], [0])
+                       for r, s in zip(reqs, plan.items)]
+            logits = runner.step(entries, download=False, tokens_from=tokens_from)
+            ids = sampler.sample_deferred(logits, i)
+            pending.append(ids)
+            tokens_from = ids.device_ptr
+            done += sch.on_step_done(plan, {r.request_id: None for r in reqs})
+            self._stats.steps += 1
+            if i + 1 == length:
+                break
+            plan = sch.schedule()
+            same = (not plan.preempted and not plan.failed and [s.request for s in plan.items] == reqs
+                    and all(s.count == 1 and s.sample for s in plan.items))
+            if not same:                       # pages ran short: look at the ids before going on
+                self._next_plan = plan
+                break
+        # the ids arrive: put them where the placeholders are, and end what a stop token ends
+        stopped = set()
+        for i, ids in enumerate(pending):
+            for r, n0, tok in zip(reqs, first_len, ids.result()):
+                if r.request_id in stopped:
+                    continue
+                r.output_tokens[n0 + i] = tok
+                if r.params.stop_tokens and tok in r.params.stop_tokens:
+                    stopped.add(r.request_id)
+                    if sch.finish_at(r, n0 + i + 1, FinishReason.STOP):
+                        done.append(r)
+        if self._next_plan is not None and stopped:
+            self._next_plan.items = [s for s in self._next_plan.items if s.request.request_id not in stopped]
+        self._stats.generated_tokens += sum(len(r.output_tokens) - n0 for r, n0 in zip(reqs, first_len))
+        self._stats.preemptions = sch.num_preemptions
+        return done
 
     def run(self) -> None:
         t0 = time.monotonic()

@@ -324,7 +324,7 @@ class StepRunner:
             b *= 2
         return b if b <= self.max_seqs else 0
 
-    def _graph_step(self, entries, bucket: int):
+    def _graph_step(self, entries, bucket: int, tokens_from=None):
         """One token for each request through the graph of this bucket.  The first step of
         a bucket runs eagerly (it sizes the arena), the second is captured, later ones
         replay.  Kernel arguments are fixed by the bucket: rows beyond the batch are
@@ -336,6 +336,8 @@ class StepRunner:
         logit_rows[n_rows:] = 0
         self.rt.copy_h2d_async(self.meta_dev.ptr, self.meta_host.ptr, words * 4)
         self.rt.record(self.meta_copied)
+        if tokens_from is not None:
+            self.rt.copy_d2d(self.meta_dev.ptr + off["tokens"] * 4, tokens_from, R * 4)
         if self.graph_logits is None:
             self.graph_logits = self.rt.empty((self.max_seqs, self.vocab), F32)
         out = self.graph_logits.rows(0, bucket)
@@ -362,9 +364,13 @@ class StepRunner:
         self.rt.graph_launch(graph)
         return self.graph_logits.rows(0, n_rows)
 
-    def step(self, entries: Sequence[StepEntry], download: bool = True):
+    def step(self, entries: Sequence[StepEntry], download: bool = True, tokens_from: Optional[int] = None):
         """Run one step.  Returns float32 logits [wanted, vocab] on the host
-        (``download=False``: the device tensor, valid until the next step)."""
+        (``download=False``: the device tensor, valid until the next step).
+        ``tokens_from``: a device pointer to int32 token ids, one per entry in the order of the
+        entries, for a step in which every entry brings one token: the ids the last step's
+        sampling kernel left on the device are fed without a trip to the host (the entries'
+        own token values are then placeholders)."""
         entries = [e for e in entries if len(e.tokens) > 0]
         if not entries:
             return np.zeros((0, self.vocab), np.float32) if download else None
@@ -391,15 +397,19 @@ class StepRunner:
             if not m.reserve(e.req, upto):
                 raise OutOfPages(f"request {e.req!r} needs pages for {upto} tokens and the pool "
                                  f"cannot give them: {m.stats()}")
+        if tokens_from is not None and T != R:
+            raise ValueError("tokens_from serves steps in which every request brings one token")
         self.rt.wait_event(self.meta_copied)     # the last step's copy has left the host buffer
         bucket = self._graph_bucket(entries)
         if bucket:
-            out = self._graph_step(entries, bucket)
+            out = self._graph_step(entries, bucket, tokens_from)
         else:
             off, words, T, R, n_rows, host_entries, max_q, max_ctx, n_multi = self._pack(entries, T, R)
             self._ensure_logits(n_rows)
             self.rt.copy_h2d_async(self.meta_dev.ptr, self.meta_host.ptr, words * 4)
             self.rt.record(self.meta_copied)
+            if tokens_from is not None:
+                self.rt.copy_d2d(self.meta_dev.ptr + off["tokens"] * 4, tokens_from, R * 4)
             ctx = self._context(off, T, R, host_entries, max_q, max_ctx, n_multi)
             self.arena.reset()
             out = self.logits.rows(0, n_rows)

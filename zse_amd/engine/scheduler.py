@@ -32,6 +32,9 @@ from ..cache.slots import OutOfSlots
 from .request import FinishReason, Request, RequestState
 
 
+UNKNOWN_TOKEN = -1      # stands in an output for a token that has not reached the host yet
+
+
 @dataclass
 class SchedulerConfig:
     max_batch_tokens: int = 4096
@@ -180,11 +183,12 @@ class Scheduler:
             self.manager.commit(req.request_id, req.num_computed)
             if not s.sample:
                 continue
-            tok = int(sampled[req.request_id])
+            known = sampled[req.request_id] is not None
+            tok = int(sampled[req.request_id]) if known else UNKNOWN_TOKEN     # still on the device: set later
             req.output_tokens.append(tok)
             req.state = RequestState.DECODING
             reason = None
-            if req.params.stop_tokens and tok in req.params.stop_tokens:
+            if known and req.params.stop_tokens and tok in req.params.stop_tokens:
                 reason = FinishReason.STOP
             elif len(req.output_tokens) >= req.params.max_tokens:
                 reason = FinishReason.LENGTH
@@ -198,6 +202,20 @@ class Scheduler:
                 self.finished[req.request_id] = req
                 done.append(req)
         return done
+
+    def finish_at(self, req: Request, length: int, reason: FinishReason) -> bool:
+        """A token that was still unknown when the request was stepped on turned out to end
+        it: cut its output to ``length`` tokens and finish it now.  Returns True if the request
+        was still running."""
+        del req.output_tokens[length:]
+        was_running = req in self.running
+        if was_running:
+            self.manager.release(req.request_id)
+            self.running.remove(req)
+            self.finished[req.request_id] = req
+        req.state = RequestState.FINISHED
+        req.finish_reason = reason
+        return was_running
 
     def stats(self) -> dict:
         return {"waiting": len(self.waiting), "running": len(self.running),

@@ -345,6 +345,12 @@ class Runtime:
             return (a.astype(np.uint32) << 16).view(np.float32)
         return a.astype(np.float32, copy=False)
 
+    def copy_d2h_async(self, host_ptr: int, src_ptr: int, nbytes: int):
+        """Enqueue a copy into pinned host memory; the data is there once an event recorded
+        after it has passed."""
+        if nbytes:
+            self._check(self.lib.zrt_d2h(host_ptr, src_ptr, nbytes, self.stream, 1), "d2h")
+
     def sync(self):
         self._check(self.lib.zrt_stream_sync(self.stream), "stream sync")
 

@@ -111,6 +111,17 @@ def sample_host(logits: np.ndarray, params: SamplingParams, u: float, past: Iter
 
 # ---------------------------------------------------------------- device sampling
 
+class PendingIds:
+    """Token ids chosen on the device, on their way to the host."""
+
+    def __init__(self, rt, device_ptr: int, host, event: int, n: int):
+        self.rt, self.device_ptr, self.host, self.event, self.n = rt, device_ptr, host, event, n
+
+    def result(self) -> List[int]:
+        self.rt.wait_event(self.event)
+        return [int(x) for x in self.host.array(0, self.n, np.int32)]
+
+
 class DeviceSampler:
     """Runs the argmax and inverse-CDF kernels on logits that are still on the device."""
 
@@ -124,6 +135,54 @@ class DeviceSampler:
         self.temp = rt.empty((max_rows,), F32)
         self.u = rt.empty((max_rows,), F64)
         self.scratch = rt.empty((max_rows * 128,), F32)     # slices of the two-stage argmax
+
+    # ---- a run of steps without waiting for the host in between
+    RING = 16       # results that may be on their way to the host at a time
+
+    def can_defer(self, rows: Sequence[dict]) -> bool:
+        """True when ``sample_deferred`` serves these rows: all on the device, all greedy or
+        all drawn with a temperature."""
+        if not rows or len(rows) > self.max_rows or not all(r["params"].on_device for r in rows):
+            return False
+        kinds = {bool(r["params"].greedy) for r in rows}
+        return len(kinds) == 1
+
+    def prepare_run(self, rows: Sequence[dict], us: Sequence[Sequence[float]]):
+        """For a run of steps over the same rows: temperatures once, and the uniform numbers
+        of every step of the run (``us[step][row]``), so that no step of the run copies
+        anything from the host."""
+        from ..runtime.device import F64
+        n = len(rows)
+        self._run_greedy = bool(rows[0]["params"].greedy)
+        if self._run_greedy:
+            return
+        self.rt.copy_h2d(self.temp.ptr, np.array([r["params"].temperature for r in rows], dtype=np.float32))
+        flat = np.ascontiguousarray(np.asarray(us, dtype=np.float64).reshape(len(us), n))
+        if getattr(self, "_run_u", None) is None or self._run_u.shape[0] < flat.size:
+            self._run_u = self.rt.empty((max(flat.size, self.max_rows * 8),), F64)
+        self.rt.copy_h2d(self._run_u.ptr, flat)
+
+    def sample_deferred(self, logits, step_in_run: int) -> "PendingIds":
+        """Enqueue the sampling of one step of a prepared run.  The ids stay on the device
+        (``.device_ptr``, valid until the next call) and travel to the host behind the
+        kernels; ``.result()`` waits for them."""
+        n, V = logits.shape
+        rt, k = self.rt, self.k
+        if self._run_greedy:
+            k.zk_argmax(logits.ptr, self.ids.ptr, n, V, self.scratch.ptr, rt.stream)
+            dev = self.ids
+        else:
+            k.zk_sample(logits.ptr, self.temp.ptr, self._run_u.ptr + step_in_run * n * 8, None, self.ids2.ptr,
+                        n, V, rt.stream)
+            dev = self.ids2
+        if getattr(self, "_ring", None) is None:
+            self._ring = [(rt.pinned(self.max_rows * 4), rt.event()) for _ in range(self.RING)]
+            self._ring_at = 0
+        host, ev = self._ring[self._ring_at % self.RING]
+        self._ring_at += 1
+        rt.copy_d2h_async(host.ptr, dev.ptr, n * 4)
+        rt.record(ev)
+        return PendingIds(rt, dev.ptr, host, ev, n)
 
     def sample(self, logits, rows: Sequence[dict]) -> List[int]:
         """``logits``: device float32 [n, vocab]; ``rows``: per row a dict with
