@@ -472,6 +472,52 @@ def test_rope_and_cache_write(rt, dtype, T, nh, nkv, hd, rot, bs, vt):
     assert np.abs(kc - want_k).max() < tol and np.array_equal(vc, want_v)
 
 
+@pytest.mark.parametrize("M,K,nh,nkv,hd,bs,vt,strip", [(5, 96, 6, 1, 32, 8, 1, 1), (16, 200, 3, 3, 64, 16, 0, 0),
+                                                        (8, 2304, 8, 4, 256, 16, 1, 1), (1, 2048, 2, 2, 96, 4, 1, 1),
+                                                        (3, 160, 4, 0, 32, 4, 1, 1), (11, 64, 5, 5, 160, 8, 0, 1),
+                                                        (7, 96, 3, 1, 48, 8, 1, 1), (9, 72, 2, 1, 16, 4, 0, 0)])
+def test_qkv_product_that_rotates_and_stores(rt, M, K, nh, nkv, hd, bs, vt, strip):
+    """The fused product of decoded tokens leaves the same bits as the product followed by the
+    rotation kernel: in q, and in the cache (which starts from a pattern, so that a store to a
+    wrong place shows as well as a missing one)."""
+    k = rt.kernels("bfloat16")
+    rng = np.random.default_rng(M * 1000 + hd)
+    N = (nh + 2 * nkv) * hd
+    pages = 7
+    a = bf16(rng.normal(size=(M, K)).astype(np.float32))
+    w = bf16(rng.normal(size=(N, K)).astype(np.float32) / math.sqrt(K))
+    pos = np.concatenate([[8191, 0, 1000], rng.integers(0, 8192, 16)])[:M].astype(np.int32)
+    slots = rng.permutation(pages * bs)[:M].astype(np.int32)
+    if M > 2:
+        slots[2] = -1
+    inv = (1.0 / 10000.0 ** (2.0 * np.arange(hd // 2) / hd)).astype(np.float32)
+    A, W = up(rt, a, "bfloat16"), up(rt, w, "bfloat16")
+    WS = W
+    if strip:
+        WS = rt.empty(((N + 15) // 16 * 16, K), "bfloat16")
+        k.zk_strip_layout(W.ptr, WS.ptr, N, K, rt.stream)
+    P, S, I = rt.upload(pos), rt.upload(slots), rt.upload(inv)
+    pattern = bf16(rng.normal(size=(pages, max(nkv, 1), bs, hd)).astype(np.float32))
+    assert k.zk_qkv_rope_bf16_supports(M, K, hd, hd)
+    got = []
+    for fused in (False, True):
+        Q = up(rt, np.zeros((M, N), np.float32), "bfloat16")
+        KC = up(rt, pattern, "bfloat16")
+        VC = up(rt, pattern.reshape(pages, max(nkv, 1), hd, bs) if vt else pattern, "bfloat16")
+        if fused:
+            k.zk_qkv_rope_bf16(A.ptr, K, WS.ptr, Q.ptr, N, M, K, strip, P.ptr, S.ptr if nkv else None, I.ptr,
+                               KC.ptr, VC.ptr, nh, nkv, hd, bs, vt, rt.stream)
+        else:
+            k.zk_gemm_bf16(A.ptr, K, WS.ptr, Q.ptr, N, 0, M, N, K, 0, 0.0, strip, None, 0, rt.stream)
+            k.zk_rope_cache_write(Q.ptr, P.ptr, S.ptr if nkv else None, I.ptr, hd, KC.ptr, VC.ptr, M, nh, nkv, hd,
+                                  bs, vt, rt.stream)
+        got.append((rt.download_f32(Q)[:, :nh * hd], rt.download_f32(KC), rt.download_f32(VC)))
+    for x, y in zip(*got):
+        assert np.array_equal(x, y)
+    assert not k.zk_qkv_rope_bf16_supports(17, K, hd, hd) and not k.zk_qkv_rope_bf16_supports(M, K, 40, 40)
+    assert not k.zk_qkv_rope_bf16_supports(M, K, hd, hd // 2)
+
+
 def test_convert_and_fill(rt):
     rng = np.random.default_rng(0)
     x = rng.normal(size=1003).astype(np.float32)

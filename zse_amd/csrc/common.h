@@ -30,6 +30,14 @@ __device__ __forceinline__ float from_f32<float>(float x) { return x; }
 template <>
 __device__ __forceinline__ __bf16 from_f32<__bf16>(float x) { return (__bf16)x; }
 
+// One rotation of a pair by an angle, written so that every kernel that rotates rounds alike
+// (a token's values must not depend on how many tokens the step holds or on which kernel took
+// it): a product rounded, then one fused multiply-add.
+__device__ __forceinline__ void rotate_pair(float a, float b, float sn, float cs, float& ra, float& rb) {
+  ra = __fmaf_rn(a, cs, -__fmul_rn(b, sn));
+  rb = __fmaf_rn(b, cs, __fmul_rn(a, sn));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = ZSE_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, ZSE_WAVE);

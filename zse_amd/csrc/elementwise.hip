@@ -272,12 +272,6 @@ __global__ void softcap_kernel(float* __restrict__ z, size_t n, float cap) {
 // rotated and stored, v is stored, at slot = page * bs + offset of the token
 // (slot < 0: nothing stored).  Cache layout per layer: K [page][kv head][bs][hd];
 // V the same, or transposed [page][kv head][hd][bs] when v_transposed is set.
-// One rotation, written so that both kernels below round alike (a token's values must not
-// depend on how many tokens the step holds): a product rounded, then one fused multiply-add.
-__device__ __forceinline__ void rotate_pair(float a, float b, float sn, float cs, float& ra, float& rb) {
-  ra = __fmaf_rn(a, cs, -__fmul_rn(b, sn));
-  rb = __fmaf_rn(b, cs, __fmul_rn(a, sn));
-}
 
 __global__ void rope_cache_write_kernel(act_t* __restrict__ qkv, const int* __restrict__ positions,
                                         const int* __restrict__ slot_map,

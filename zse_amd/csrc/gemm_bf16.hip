@@ -44,18 +44,45 @@ __device__ __forceinline__ bf16x8 zero8() {
 }
 
 // ------------------------------------------------------------------ skinny
+// What the q|k|v product of decoded tokens does with its results instead of storing them all:
+// q and k heads are rotated (pairs (i, i + hd/2), angle position * inv_freq[i]), q goes to C,
+// k and v to the token's place in the paged cache.
+struct RopeStore {
+  const int* positions;
+  const int* slot_map;  // null: nothing is stored in the cache (nkv = 0)
+  const float* inv_freq;
+  __bf16* kcache;
+  __bf16* vcache;
+  int nh, nkv, hd, bs, v_transposed;
+};
+
+__device__ __forceinline__ void store4(__bf16* dst, const float (&x)[4]) {
+  bf16x4 o;
+#pragma unroll
+  for (int i = 0; i < 4; i++) o[i] = (__bf16)x[i];
+  *(bf16x4*)dst = o;
+}
+
 // GATED: the block also streams the strip of "up" rows I + n and stores act(g)*u.
-template <int MT, bool GATED, int NW>
+// ROPE (M <= 16): W is [(nh + 2 nkv) hd, K]; the block's 16 weight rows are eight places of a
+// head's first half and their partners in the rotation, hd/2 rows further on, so that partners
+// meet in lanes 32 apart; the results are finished as RopeStore says.  Every result is rounded
+// to 16 bits before it is rotated, as the separate product and rotation kernels do, so a
+// token's keys are the same bits whichever way it came.
+template <int MT, bool GATED, int NW, bool ROPE = false>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __restrict__ A, int lda,
                                                           const __bf16* __restrict__ W,
                                                           void* __restrict__ C, int ldc, int c_is_f32,
                                                           int M, int N, int K, int epi, float cap,
-                                                          int w_strip) {
+                                                          int w_strip, RopeStore rs) {
+  static_assert(!ROPE || (MT == 1 && !GATED), "the rotating epilogue takes up to 16 rows");
   constexpr int NS = GATED ? 2 : 1;
   __shared__ f32x4 red[NW - 1][NS][MT][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, kq = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  // the block's strips of 16 weight rows
+  const int strip0 = blockIdx.x, strip1 = N / 16 + blockIdx.x;
+  const int n0 = strip0 * 16;
   // Row-major weights: a lane reads row n0 + r at 8 * kq, a 32-wide step further on is 32
   // elements away.  Strip layout: the 64 lanes' pieces of one (strip, step) are one
   // contiguous KB, a step further on is 512 elements away, strips follow each other.
@@ -63,10 +90,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
   const int ksteps = (K + 31) / 32;
   const size_t wstep = w_strip ? 512 : 32;
   const __bf16* wp[NS];
-  wp[0] = w_strip ? W + (size_t)blockIdx.x * ksteps * 512 + lane * 8 : W + (size_t)wrow * K + kq * 8;
+  wp[0] = w_strip ? W + (size_t)strip0 * ksteps * 512 + lane * 8 : W + (size_t)wrow * K + kq * 8;
   if (GATED)
-    wp[NS - 1] = w_strip ? W + ((size_t)(N / 16) + blockIdx.x) * ksteps * 512 + lane * 8
+    wp[NS - 1] = w_strip ? W + (size_t)strip1 * ksteps * 512 + lane * 8
                          : W + (size_t)(N + wrow) * K + kq * 8;
+  int head = 0, hpos = 0;  // ROPE: the head and the first of the block's eight places in its first half
+  if (ROPE) {
+    const int per_head = rs.hd / 16;
+    head = blockIdx.x / per_head;
+    hpos = (blockIdx.x % per_head) * 8;
+    const int row = head * rs.hd + hpos + (r < 8 ? r : rs.hd / 2 + r - 8);
+    wp[0] = w_strip ? W + (size_t)(row / 16) * ksteps * 512 + (16 * kq + row % 16) * 8
+                    : W + (size_t)row * K + kq * 8;
+  }
   const __bf16* ap[MT];
   bool av[MT];
 #pragma unroll
@@ -110,6 +146,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
   };
   bf16x8 wf0[NS][STEPS], af0[MT][STEPS], wf1[NS][STEPS], af1[MT][STEPS];
   if (s_begin < s_end) fetch(s_begin, wf0, af0);
+  // the angles of the lane's four pairs, worked out while the first loads are on their way
+  float sn[4], cs[4];
+  if (ROPE && wave == 0 && head < rs.nh + rs.nkv) {
+    const float pos = (float)rs.positions[min(r, M - 1)];
+#pragma unroll
+    for (int i = 0; i < 4; i++) sincosf(pos * rs.inv_freq[hpos + 4 * (kq & 1) + i], &sn[i], &cs[i]);
+  }
   for (int s0 = s_begin; s0 < s_end; s0 += 2 * STEPS) {
     if (s0 + STEPS < s_end) fetch(s0 + STEPS, wf1, af1);
     multiply(wf0, af0);
@@ -135,6 +178,40 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
       v[g] = acc[g][mt];
 #pragma unroll
       for (int w = 0; w < NW - 1; w++) v[g] += red[w][g][mt][lane];
+    }
+    if (ROPE) {
+      // results 4 kq + i of the block's 16: lanes 0..31 hold places hpos + 4 kq + i of the
+      // head's first half, lanes 32..63 their partners in the second
+      const bool first = kq < 2;
+      const int half = rs.hd / 2, at = hpos + 4 * (kq & 1) + (first ? 0 : half);
+      float x[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        x[i] = (float)(__bf16)v[0][i];
+        const float y = __shfl_xor(x[i], 32);
+        if (head < rs.nh + rs.nkv) {
+          float ra, rb;
+          rotate_pair(first ? x[i] : y, first ? y : x[i], sn[i], cs[i], ra, rb);
+          x[i] = first ? ra : rb;
+        }
+      }
+      if (m >= M) continue;
+      if (head < rs.nh) {
+        store4((__bf16*)C + (size_t)m * ldc + (size_t)head * rs.hd + at, x);
+        continue;
+      }
+      const int slot = rs.slot_map ? rs.slot_map[m] : -1;
+      if (slot < 0) continue;
+      const int kvh = (head - rs.nh) % rs.nkv;
+      const size_t page = slot / rs.bs, off = slot % rs.bs;
+      if (head < rs.nh + rs.nkv || !rs.v_transposed) {
+        store4((head < rs.nh + rs.nkv ? rs.kcache : rs.vcache) + ((page * rs.nkv + kvh) * rs.bs + off) * rs.hd + at, x);
+      } else {
+        __bf16* vt = rs.vcache + (page * rs.nkv + kvh) * (size_t)rs.hd * rs.bs + off;
+#pragma unroll
+        for (int i = 0; i < 4; i++) vt[(size_t)(at + i) * rs.bs] = (__bf16)x[i];
+      }
+      continue;
     }
     if (m >= M) continue;
 #pragma unroll
@@ -630,13 +707,50 @@ static int launch_skinny(const void* A, int lda, const void* W, void* C, int ldc
   const bool wide = grid.x < 512 && K >= 2048 && mt <= 2;
 #define ZK_SKINNY(MT_, NW_)                                                                           \
   gemm_skinny_kernel<MT_, GATED, NW_><<<grid, NW_ * 64, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, \
-                                                                C, ldc, c_is_f32, M, N, K, epi, cap, w_strip)
+                                                                C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, \
+                                                                RopeStore{})
   if (mt == 1) { if (wide) ZK_SKINNY(1, 8); else ZK_SKINNY(1, 4); }
   else if (mt == 2) { if (wide) ZK_SKINNY(2, 8); else ZK_SKINNY(2, 4); }
   else if (mt == 3) ZK_SKINNY(3, 4);
   else ZK_SKINNY(4, 4);
 #undef ZK_SKINNY
   return zk_launch_status("zk_gemm_bf16 (skinny)");
+}
+
+// The q|k|v product of up to 16 decoded tokens with the rotation and the cache store as its
+// epilogue: W [(nh + 2 nkv) hd, K] (row-major or strip layout), q rotated into Q [M, ldq] at
+// columns [0, nh hd), k rotated and v as it is into the cache at slot_map[m] (a negative slot
+// stores nothing).  The same bits as zk_gemm_bf16 followed by zk_rope_cache_write.  nkv may be 0
+// (a mixer that reads another's cache); then slot_map and the caches are not used.
+extern "C" int zk_qkv_rope_bf16_supports(int M, int K, int hd, int rotary_dim) {
+  return M >= 1 && M <= 16 && K % 8 == 0 && hd % 16 == 0 && rotary_dim == hd;
+}
+
+extern "C" int zk_qkv_rope_bf16(const void* A, int lda, const void* W, void* Q, int ldq, int M, int K,
+                                int w_strip, const int* positions, const int* slot_map,
+                                const float* inv_freq, void* kcache, void* vcache, int nh, int nkv, int hd,
+                                int bs, int v_transposed, void* stream) {
+  ZK_REQUIRE(M >= 1 && M <= 16 && K > 0 && K % 8 == 0 && lda % 8 == 0 && lda >= K,
+             "zk_qkv_rope_bf16: 1 to 16 rows, K and lda multiples of 8");
+  ZK_REQUIRE(nh > 0 && nkv >= 0 && hd > 0 && hd % 16 == 0, "zk_qkv_rope_bf16: head_dim must be a multiple of 16");
+  ZK_REQUIRE(ldq >= nh * hd && ldq % 4 == 0, "zk_qkv_rope_bf16: ldq too small or not a multiple of 4");
+  ZK_REQUIRE(!w_strip || K % 32 == 0, "zk_qkv_rope_bf16: strip layout needs K % 32 == 0");
+  ZK_REQUIRE(positions && inv_freq, "zk_qkv_rope_bf16: positions and inv_freq are needed");
+  ZK_REQUIRE(nkv == 0 || (slot_map && kcache && vcache && bs > 0), "zk_qkv_rope_bf16: the cache is needed");
+  ZK_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) && ((uintptr_t)Q % 8 == 0),
+             "zk_qkv_rope_bf16: operands must be 16-byte aligned");
+  const int N = (nh + 2 * nkv) * hd;
+  RopeStore rs{positions, nkv ? slot_map : nullptr, inv_freq, (__bf16*)kcache, (__bf16*)vcache, nh, nkv, hd, bs,
+               v_transposed};
+  dim3 grid(N / 16);
+  hipStream_t s = (hipStream_t)stream;
+  if (grid.x < 512 && K >= 2048)
+    gemm_skinny_kernel<1, false, 8, true><<<grid, 512, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, Q, ldq, 0, M,
+                                                               N, K, EPI_NONE, 0.f, w_strip, rs);
+  else
+    gemm_skinny_kernel<1, false, 4, true><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, Q, ldq, 0, M,
+                                                               N, K, EPI_NONE, 0.f, w_strip, rs);
+  return zk_launch_status("zk_qkv_rope_bf16");
 }
 
 // Strip layout of a [N, K] weight matrix, K % 32 == 0: rows in strips of 16 (the last strip

@@ -17,7 +17,7 @@ from typing import List
 
 from ..runtime.device import BF16, Tensor
 from .base import PagedKV, Part, TensorReq, build_part, register_part
-from .ops import linear
+from .ops import linear, tuned_gemm
 
 
 class PagedAttention(Part):
@@ -68,17 +68,27 @@ class PagedAttention(Part):
         nh, nkv, hd = s.num_heads, s.num_kv_heads, s.head_dim
         n_store = 0 if self.shared_kv else nkv
         width = (nh + 2 * n_store) * hd
-        qkv = linear(ctx, x, self.w_qkv, ctx.alloc((T, width)))
         g = ctx.group(cache.group)
         tables = self.position.rotary_tables()
-        if tables is None:
-            self.position.apply(ctx, qkv, nh, n_store, hd)
-            inv_freq, rotary_dim = 0, 0
+        if (tables is not None and tuned_gemm(ctx, s.hidden_size) and k.has("zk_qkv_rope_bf16")
+                and k.zk_qkv_rope_bf16_supports(T, s.hidden_size, hd, tables[1])):
+            # few decoded tokens: the product rotates and stores its own results
+            qkv = ctx.alloc((T, width))
+            k.zk_qkv_rope_bf16(x.ptr, s.hidden_size, self.w_qkv.ptr, qkv.ptr, width, T, s.hidden_size,
+                               1 if self.w_qkv.layout == "strip" else 0, ctx.positions,
+                               None if self.shared_kv else g.slot_map, tables[0].ptr, cache.k.ptr,
+                               cache.v.ptr, nh, n_store, hd, g.page_size, 1 if cache.v_transposed else 0,
+                               ctx.stream)
         else:
-            inv_freq, rotary_dim = tables[0].ptr, tables[1]
-        k.zk_rope_cache_write(qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map,
-                              inv_freq or None, rotary_dim, cache.k.ptr, cache.v.ptr, T, nh, n_store,
-                              hd, g.page_size, 1 if cache.v_transposed else 0, ctx.stream)
+            qkv = linear(ctx, x, self.w_qkv, ctx.alloc((T, width)))
+            if tables is None:
+                self.position.apply(ctx, qkv, nh, n_store, hd)
+                inv_freq, rotary_dim = 0, 0
+            else:
+                inv_freq, rotary_dim = tables[0].ptr, tables[1]
+            k.zk_rope_cache_write(qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map,
+                                  inv_freq or None, rotary_dim, cache.k.ptr, cache.v.ptr, T, nh, n_store,
+                                  hd, g.page_size, 1 if cache.v_transposed else 0, ctx.stream)
         o = ctx.alloc((T, nh * hd))
         cap = float(s.softcap) if s.softcap else 0.0
         win = int(s.window) if s.window else 0
