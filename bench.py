@@ -100,9 +100,10 @@ def main():
     points = sorted({int(x) for x in a.points.split(",") if x} | {a.batch})
     max_b = max(points)
     page = 16
+    longest = max(a.context, a.prefill_tokens)       # a prompt longer than the decode context still fits
     runner = StepRunner(model, rt, "bfloat16", page_size=page,
-                        num_pages=max_b * (-(-a.context // page) + 1) + 8, max_seqs=max_b,
-                        max_batch_tokens=max(a.prefill_tokens, max_b), max_model_len=a.context,
+                        num_pages=max(max_b * (-(-a.context // page) + 1), -(-longest // page)) + 8, max_seqs=max_b,
+                        max_batch_tokens=max(a.prefill_tokens, max_b), max_model_len=longest,
                         use_graphs=not a.no_graphs)
     sampler = DeviceSampler(rt, runner.k, max_b)
     greedy = SamplingParams(temperature=0.0)

@@ -84,17 +84,17 @@ def test_gemm_bf16_matrix_cores(rt, M, N, K):
     A, W = up(rt, a, "bfloat16"), up(rt, w, "bfloat16")
     want = a.astype(np.float64) @ w.astype(np.float64).T
     C = rt.empty((M, N), "float32")
-    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, N, 1, M, N, K, 0, 0.0, 0, None, 0, rt.stream)
+    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, N, 1, M, N, K, 0, 0.0, 0, None, 0, None, rt.stream)
     assert np.abs(rt.download(C) - want).max() < 1e-4 * math.sqrt(K)      # float accumulation
     ws = gemm_workspace(rt)      # with a workspace a long K is split over blocks and joined
     C2 = rt.empty((M, N), "float32")
-    k.zk_gemm_bf16(A.ptr, K, W.ptr, C2.ptr, N, 1, M, N, K, 0, 0.0, 0, ws.ptr, ws.nbytes, rt.stream)
+    k.zk_gemm_bf16(A.ptr, K, W.ptr, C2.ptr, N, 1, M, N, K, 0, 0.0, 0, ws.ptr, ws.nbytes, None, rt.stream)
     assert np.abs(rt.download(C2) - want).max() < 1e-4 * math.sqrt(K)
     Cb = rt.empty((M, N), "bfloat16")
-    k.zk_gemm_bf16(A.ptr, K, W.ptr, Cb.ptr, N, 0, M, N, K, 0, 0.0, 0, None, 0, rt.stream)
+    k.zk_gemm_bf16(A.ptr, K, W.ptr, Cb.ptr, N, 0, M, N, K, 0, 0.0, 0, None, 0, None, rt.stream)
     got = rt.download_f32(Cb)
     assert np.abs(got - want).max() <= np.abs(want).max() * 2.0 ** -8 + 1e-4 * math.sqrt(K)
-    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, N, 1, M, N, K, 1, 7.5, 0, None, 0, rt.stream)
+    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, N, 1, M, N, K, 1, 7.5, 0, None, 0, None, rt.stream)
     assert np.abs(rt.download(C) - 7.5 * np.tanh(want / 7.5)).max() < 1e-4 * math.sqrt(K)
 
 
@@ -106,7 +106,7 @@ def test_gemm_bf16_gated_epilogue(rt, M, I, K, act):
     a, w = bf16(rng.normal(size=(M, K))), bf16(rng.normal(size=(2 * I, K)) * 0.3)
     A, W = up(rt, a, "bfloat16"), up(rt, w, "bfloat16")
     C = rt.empty((M, I), "float32")
-    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, I, 1, M, I, K, 2 if act == "gelu_tanh" else 3, 0.0, 0, None, 0, rt.stream)
+    k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, I, 1, M, I, K, 2 if act == "gelu_tanh" else 3, 0.0, 0, None, 0, None, rt.stream)
     g = a.astype(np.float64) @ w[:I].astype(np.float64).T
     u = a.astype(np.float64) @ w[I:].astype(np.float64).T
     want = (gelu(g) if act == "gelu_tanh" else g / (1 + np.exp(-g))) * u
@@ -136,21 +136,21 @@ def test_gemm_bf16_strip_layout(rt, M, N, K, gated):
     C = rt.empty((M, N), "float32")
     ws = gemm_workspace(rt)
     if gated:
-        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 2, 0.0, 1, ws.ptr, ws.nbytes, rt.stream)
+        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 2, 0.0, 1, ws.ptr, ws.nbytes, None, rt.stream)
         g = a.astype(np.float64) @ w[:N].astype(np.float64).T
         want = gelu(g) * (a.astype(np.float64) @ w[N:].astype(np.float64).T)
         tol = 2e-4 * math.sqrt(K) * max(1.0, np.abs(want).max())
     else:
-        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 0, 0.0, 1, ws.ptr, ws.nbytes, rt.stream)
+        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 0, 0.0, 1, ws.ptr, ws.nbytes, None, rt.stream)
         want = a.astype(np.float64) @ w.astype(np.float64).T
         tol = 1e-4 * math.sqrt(K)
     got = rt.download(C)
     assert np.abs(got - want).max() < tol
     # a second launch, over the first one's leavings in the workspace, gives the same bits
-    k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 2 if gated else 0, 0.0, 1, ws.ptr, ws.nbytes, rt.stream)
+    k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 2 if gated else 0, 0.0, 1, ws.ptr, ws.nbytes, None, rt.stream)
     assert np.array_equal(rt.download(C), got)
     if 16 < M <= 64:   # without a workspace K is not split over blocks: same values beyond rounding
-        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 2 if gated else 0, 0.0, 1, None, 0, rt.stream)
+        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 2 if gated else 0, 0.0, 1, None, 0, None, rt.stream)
         assert np.abs(rt.download(C) - want).max() < tol
     if not gated and K % 32 == 0:
         toks = rng.integers(0, N, 5).astype(np.int32)
@@ -183,7 +183,7 @@ def test_gemm_bf16_random_shapes(rt):
         C = rt.empty((M, N), "float32")
         use_ws = bool(rng.integers(0, 2))
         k.zk_gemm_bf16(A.ptr, K, W.ptr, C.ptr, N, 1, M, N, K, 2 if gated else 0, 0.0, 1 if strip else 0,
-                       ws.ptr if use_ws else None, ws.nbytes if use_ws else 0, rt.stream)
+                       ws.ptr if use_ws else None, ws.nbytes if use_ws else 0, None, rt.stream)
         if gated:
             g = a.astype(np.float64) @ w[:N].astype(np.float64).T
             want = gelu(g) * (a.astype(np.float64) @ w[N:].astype(np.float64).T)
@@ -193,6 +193,49 @@ def test_gemm_bf16_random_shapes(rt):
             tol = 1e-4 * math.sqrt(K)
         err = np.abs(rt.download(C) - want).max()
         assert err < tol, f"case {case}: M={M} N={N} K={K} strip={strip} gated={gated} workspace={use_ws}: {err}"
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 2304, 2048), (1, 2304, 9216), (16, 1024, 4096), (40, 2304, 9216), (64, 4096, 2304),
+                                   (17, 1536, 1024)])
+def test_gemm_bf16_leaves_partial_sums_to_a_reader_that_asks(rt, M, N, K):
+    """A caller that passes a place for the number of parts gets the split product's partial
+    sums as planes of [M, N] floats; added in order and rounded they are the bits the product
+    stores when it joins them itself.  A product that does not split K says 0 and fills C."""
+    import ctypes
+    k = rt.kernels("bfloat16")
+    rng = np.random.default_rng(M + N)
+    a = bf16(rng.normal(size=(M, K)).astype(np.float32))
+    w = bf16(rng.normal(size=(N, K)).astype(np.float32) / math.sqrt(K))
+    A, W = up(rt, a, "bfloat16"), up(rt, w, "bfloat16")
+    WS = rt.empty((N, K), "bfloat16")
+    k.zk_strip_layout(W.ptr, WS.ptr, N, K, rt.stream)
+    ws = gemm_workspace(rt)
+    C = rt.zeros((M, N), "bfloat16")
+    k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 0, M, N, K, 0, 0.0, 1, ws.ptr, ws.nbytes, None, rt.stream)
+    joined = rt.download_f32(C)
+    want = a.astype(np.float64) @ w.astype(np.float64).T
+    assert np.abs(joined - want).max() <= 2.0 ** -7 * max(1.0, np.abs(want).max())
+    C2 = rt.zeros((M, N), "bfloat16")
+    parts = ctypes.c_int(-1)
+    k.zk_gemm_bf16(A.ptr, K, WS.ptr, C2.ptr, N, 0, M, N, K, 0, 0.0, 1, ws.ptr, ws.nbytes, ctypes.byref(parts), rt.stream)
+    P = parts.value
+    assert P >= 0
+    if P == 0:
+        assert np.array_equal(rt.download_f32(C2), joined)
+        return
+    planes = rt.download(ws)[:P * M * N].reshape(P, M, N)
+    total = planes[0].copy()
+    for p in range(1, P):
+        total = total + planes[p]
+    if M > 16:
+        assert np.array_equal(bf16(total), joined)             # the same split either way
+    else:
+        assert np.abs(bf16(total) - want).max() <= 2.0 ** -7 * max(1.0, np.abs(want).max())
+    assert not rt.download_f32(C2).any()                       # C was left alone
+    # a float result, an epilogue or rows longer than N are joined by the product itself
+    C3 = rt.zeros((M, N), "float32")
+    k.zk_gemm_bf16(A.ptr, K, WS.ptr, C3.ptr, N, 1, M, N, K, 0, 0.0, 1, ws.ptr, ws.nbytes, ctypes.byref(parts), rt.stream)
+    assert parts.value == 0 and np.abs(rt.download(C3) - want).max() <= 1e-3 * max(1.0, np.abs(want).max())
 
 
 def test_gemm_reference_vector(rt):
@@ -210,7 +253,7 @@ def test_gemm_refuses_what_it_cannot_do(rt):
     k = rt.kernels("bfloat16")
     A, W, C = rt.empty((4, 100), "bfloat16"), rt.empty((8, 100), "bfloat16"), rt.empty((4, 8), "float32")
     with pytest.raises(DeviceError, match="multiples of 8"):
-        k.zk_gemm_bf16(A.ptr, 100, W.ptr, C.ptr, 8, 1, 4, 8, 100, 0, 0.0, 0, None, 0, rt.stream)
+        k.zk_gemm_bf16(A.ptr, 100, W.ptr, C.ptr, 8, 1, 4, 8, 100, 0, 0.0, 0, None, 0, None, rt.stream)
 
 
 # ------------------------------------------------------------------ attention over the cache
@@ -382,15 +425,27 @@ def test_rmsnorm_and_the_fused_joins(rt, dtype, T, H, eps, uo):
     h = rng.normal(size=(T, H)).astype(np.float32)
     Hd = rt.upload(h)
     nxt = rt.empty((T, H), dtype)
-    k.zk_norm_add_norm(ptr(up(rt, sub, dtype)), W.ptr, eps, uo, Hd.ptr, W2.ptr, eps * 2, uo, nxt.ptr, T, H, rt.stream)
+    k.zk_norm_add_norm(ptr(up(rt, sub, dtype)), 0, W.ptr, eps, uo, Hd.ptr, W2.ptr, eps * 2, uo, nxt.ptr, T, H, rt.stream)
     h_want = h.astype(np.float64) + norm(sub.astype(np.float64), w)
     assert np.abs(rt.download(Hd) - h_want).max() < 1e-5 * max(1, np.abs(h_want).max())     # the stream stays float
     x_want = h_want / np.sqrt((h_want * h_want).mean(-1, keepdims=True) + eps * 2) * gain(w2)
     assert np.abs(rt.download_f32(nxt) - x_want).max() <= tol * np.abs(x_want).max()
     # no post norm: a plain residual sum; no next norm: nothing else is written
     Hd2 = rt.upload(h)
-    k.zk_norm_add_norm(ptr(up(rt, sub, dtype)), None, 0.0, 0, Hd2.ptr, None, 0.0, 0, None, T, H, rt.stream)
+    k.zk_norm_add_norm(ptr(up(rt, sub, dtype)), 0, None, 0.0, 0, Hd2.ptr, None, 0.0, 0, None, T, H, rt.stream)
     assert np.abs(rt.download(Hd2) - (h.astype(np.float64) + sub)).max() < 1e-6
+    # the sublayer's output as three planes of partial sums: the same bits as their sum, rounded
+    # to the activation type, gives when handed over as one tensor
+    planes = rng.normal(size=(3, T, H)).astype(np.float32)
+    total = (planes[0] + planes[1]) + planes[2]
+    if dtype == "bfloat16":
+        total = bf16(total)
+    got = []
+    for src, parts in ((up(rt, total, dtype), 0), (rt.upload(planes), 3)):
+        Hd3, nxt3 = rt.upload(h), rt.empty((T, H), dtype)
+        k.zk_norm_add_norm(src.ptr, parts, W.ptr, eps, uo, Hd3.ptr, W2.ptr, eps * 2, uo, nxt3.ptr, T, H, rt.stream)
+        got.append((rt.download(Hd3), rt.download_f32(nxt3)))
+    assert np.array_equal(got[0][0], got[1][0]) and np.array_equal(got[0][1], got[1][1])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -508,7 +563,7 @@ def test_qkv_product_that_rotates_and_stores(rt, M, K, nh, nkv, hd, bs, vt, stri
             k.zk_qkv_rope_bf16(A.ptr, K, WS.ptr, Q.ptr, N, M, K, strip, P.ptr, S.ptr if nkv else None, I.ptr,
                                KC.ptr, VC.ptr, nh, nkv, hd, bs, vt, rt.stream)
         else:
-            k.zk_gemm_bf16(A.ptr, K, WS.ptr, Q.ptr, N, 0, M, N, K, 0, 0.0, strip, None, 0, rt.stream)
+            k.zk_gemm_bf16(A.ptr, K, WS.ptr, Q.ptr, N, 0, M, N, K, 0, 0.0, strip, None, 0, None, rt.stream)
             k.zk_rope_cache_write(Q.ptr, P.ptr, S.ptr if nkv else None, I.ptr, hd, KC.ptr, VC.ptr, M, nh, nkv, hd,
                                   bs, vt, rt.stream)
         got.append((rt.download_f32(Q)[:, :nh * hd], rt.download_f32(KC), rt.download_f32(VC)))

@@ -71,20 +71,31 @@ __global__ void rmsnorm_kernel(const TIn* __restrict__ x, const int* __restrict_
     o[i] = from_f32<act_t>(to_f32(xr[i]) * rs * gain(w, i, unit_offset));
 }
 
+// One value of the sublayer's output.  parts > 0: it still lies in `parts` float planes of
+// [rows, H] partial sums (a matrix product that split K and left the adding up to its reader);
+// they are added in order and rounded to the activation type, which is what the product's own
+// joining kernel would have stored.
+__device__ __forceinline__ float sub_value(const void* __restrict__ sub, int parts, size_t plane, size_t at) {
+  if (parts <= 0) return to_f32(((const act_t*)sub)[at]);
+  float x = ((const float*)sub)[at];
+  for (int p = 1; p < parts; p++) x += ((const float*)sub)[p * plane + at];
+  return to_f32(from_f32<act_t>(x));
+}
+
 // h += N_post(sub)  (w_post null: h += sub);  then, if w_next: out = N_next(h)
-__global__ void norm_add_norm_kernel(const act_t* __restrict__ sub, const float* __restrict__ w_post,
+__global__ void norm_add_norm_kernel(const void* __restrict__ sub, int parts, const float* __restrict__ w_post,
                                      float eps_post, int uo_post, float* __restrict__ h,
                                      const float* __restrict__ w_next, float eps_next, int uo_next,
                                      act_t* __restrict__ out, int H) {
   __shared__ float red[17];
   const int r = blockIdx.x;
-  const act_t* s = sub + (size_t)r * H;
+  const size_t plane = (size_t)gridDim.x * H, row = (size_t)r * H;
   float* hr = h + (size_t)r * H;
   float rs = 1.f;
   if (w_post) {
     float ss = 0.f;
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
-      float v = to_f32(s[i]);
+      float v = sub_value(sub, parts, plane, row + i);
       ss += v * v;
     }
     ss = block_sum(ss, red);
@@ -92,7 +103,7 @@ __global__ void norm_add_norm_kernel(const act_t* __restrict__ sub, const float*
   }
   float ss2 = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float v = to_f32(s[i]);
+    float v = sub_value(sub, parts, plane, row + i);
     if (w_post) v = v * rs * gain(w_post, i, uo_post);
     v = hr[i] + v;
     hr[i] = v;
@@ -176,12 +187,14 @@ __global__ __launch_bounds__(256) void rmsnorm_fast_kernel(const TIn* __restrict
 // and more rows share a CU.
 template <int MAXV>
 __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
-    const act_t* __restrict__ sub, const float* __restrict__ w_post, float eps_post, int uo_post,
+    const void* __restrict__ sub, int parts, const float* __restrict__ w_post, float eps_post, int uo_post,
     float* __restrict__ h, const float* __restrict__ w_next, float eps_next, int uo_next,
     act_t* __restrict__ out, int H) {
   __shared__ float red[17];
   const int r = blockIdx.x;
-  const act_t* s = sub + (size_t)r * H;
+  const act_t* s = (const act_t*)sub + (size_t)r * H;
+  const float* sf = (const float*)sub + (size_t)r * H;      // parts > 0: planes of [rows, H] partial sums
+  const size_t plane = (size_t)gridDim.x * H;
   float* hr = h + (size_t)r * H;
   // every load is issued before the first sum is needed: one trip to memory, not three
   float v[MAXV][4], hv[MAXV][4], gp[MAXV][4], gn[MAXV][4];
@@ -190,7 +203,19 @@ __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
   for (int j = 0; j < MAXV; j++) {
     const int i = threadIdx.x * 4 + j * 1024;
     if (i < H) {
-      load4<act_t>(s + i, v[j]);
+      if (parts <= 0) {
+        load4<act_t>(s + i, v[j]);
+      } else {
+        load4<float>(sf + i, v[j]);
+        for (int p = 1; p < parts; p++) {
+          float t[4];
+          load4<float>(sf + p * plane + i, t);
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[j][e] += t[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[j][e] = to_f32(from_f32<act_t>(v[j][e]));
+      }
       load4<float>(hr + i, hv[j]);
       if (w_post) load4<float>(w_post + i, gp[j]);
       if (w_next) load4<float>(w_next + i, gn[j]);
@@ -481,24 +506,26 @@ int zk_rmsnorm(const void* x, int x_is_f32, const int* rows, const float* w, voi
   return zk_launch_status("zk_rmsnorm");
 }
 
-int zk_norm_add_norm(const void* sub, const float* w_post, float eps_post, int uo_post, float* h,
+// sub_parts > 0: sub holds that many float planes of [T, H] partial sums instead of [T, H]
+// values of the activation type (see sub_value).
+int zk_norm_add_norm(const void* sub, int sub_parts, const float* w_post, float eps_post, int uo_post, float* h,
                      const float* w_next, float eps_next, int uo_next, void* out, int T, int H,
                      void* stream) {
-  ZK_REQUIRE(T >= 0 && H > 0, "zk_norm_add_norm: bad sizes");
+  ZK_REQUIRE(T >= 0 && H > 0 && sub_parts >= 0, "zk_norm_add_norm: bad sizes");
   ZK_REQUIRE(w_next == nullptr || out != nullptr, "zk_norm_add_norm: next norm without output");
   if (T == 0) return 0;
   if (H % 4 == 0 && H <= NF_MAXV * 1024) {
     if (H <= 3 * 1024)
-      norm_add_norm_fast_kernel<3><<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)sub, w_post, eps_post, uo_post,
-                                                                       h, w_next, eps_next, uo_next, (act_t*)out, H);
+      norm_add_norm_fast_kernel<3><<<T, 256, 0, (hipStream_t)stream>>>(sub, sub_parts, w_post, eps_post, uo_post, h,
+                                                                       w_next, eps_next, uo_next, (act_t*)out, H);
     else
-      norm_add_norm_fast_kernel<NF_MAXV><<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)sub, w_post, eps_post,
+      norm_add_norm_fast_kernel<NF_MAXV><<<T, 256, 0, (hipStream_t)stream>>>(sub, sub_parts, w_post, eps_post,
                                                                              uo_post, h, w_next, eps_next, uo_next,
                                                                              (act_t*)out, H);
     return zk_launch_status("zk_norm_add_norm");
   }
-  norm_add_norm_kernel<<<T, 256, 0, (hipStream_t)stream>>>((const act_t*)sub, w_post, eps_post, uo_post, h,
-                                                           w_next, eps_next, uo_next, (act_t*)out, H);
+  norm_add_norm_kernel<<<T, 256, 0, (hipStream_t)stream>>>(sub, sub_parts, w_post, eps_post, uo_post, h, w_next,
+                                                           eps_next, uo_next, (act_t*)out, H);
   return zk_launch_status("zk_norm_add_norm");
 }
 

@@ -152,10 +152,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
   if (s_begin < s_end) fetch(s_begin, wf0, af0);
   // the angles of the lane's four pairs, worked out while the first loads are on their way
   float sn[4], cs[4];
-  if (ROPE && wave == 0 && head < rs.nh + rs.nkv) {
-    const float pos = (float)rs.positions[min(r, M - 1)];
+  int slot = -1;
+  if (ROPE && wave == 0) {
+    if (head >= rs.nh && rs.slot_map) slot = rs.slot_map[min(r, M - 1)];
+    if (head < rs.nh + rs.nkv) {
+      const float pos = (float)rs.positions[min(r, M - 1)];
 #pragma unroll
-    for (int i = 0; i < 4; i++) sincosf(pos * rs.inv_freq[hpos + 4 * (kq & 1) + i], &sn[i], &cs[i]);
+      for (int i = 0; i < 4; i++) sincosf(pos * rs.inv_freq[hpos + 4 * (kq & 1) + i], &sn[i], &cs[i]);
+    }
   }
   for (int s0 = s_begin; s0 < s_end; s0 += 2 * STEPS) {
     if (s0 + STEPS < s_end) fetch(s0 + STEPS, wf1, af1);
@@ -204,7 +208,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
         store4((__bf16*)C + (size_t)m * ldc + (size_t)head * rs.hd + at, x);
         continue;
       }
-      const int slot = rs.slot_map ? rs.slot_map[m] : -1;
       if (slot < 0) continue;
       const int kvh = (head - rs.nh) % rs.nkv;
       const size_t page = slot / rs.bs, off = slot % rs.bs;
@@ -557,6 +560,13 @@ static int launch_tile(const void* A, int lda, const void* W, void* C, int ldc, 
   return zk_launch_status("zk_gemm_bf16 (tile)");
 }
 
+// A caller that passes `parts` takes the partial sums of a split product as they are: planes of
+// [M, N] floats at the start of the workspace, nothing in C.  That fits a plain product into a
+// 16-bit C whose rows are N long, N a whole number of strips.
+static bool joinable_by_reader(int N, int ldc, int c_is_f32, int epi) {
+  return N % 16 == 0 && ldc == N && !c_is_f32 && epi == EPI_NONE;
+}
+
 // ------------------------------------------------------------------ mid (16 < M <= 64)
 // With more than one column tile the activations weigh more than the weights on the way
 // from L2 to the CUs when every 16-row strip fetches them again (64 rows of A per 16 rows
@@ -600,7 +610,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
                                                        const __bf16* __restrict__ W,
                                                        void* __restrict__ C, int ldc, int c_is_f32,
                                                        int M, int N, int K, int epi, float cap,
-                                                       f32x4* __restrict__ partials, int ksplit) {
+                                                       float* __restrict__ partials, int ksplit) {
   constexpr int NS = GATED ? 2 : 1;
   __shared__ __bf16 sA[2][MT * 16][GM_LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -686,66 +696,83 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
     __syncthreads();
   }
   if (ksplit > 1) {
+    // the range's partial sums: plane (range, g) of [M, npad] floats
     if (!strip_ok) return;
-    f32x4* mine = partials + (((size_t)blockIdx.x * ksplit + blockIdx.y) * 4 + wave) * (NS * MT * 64) + lane;
+    const size_t npad = (size_t)nstrips * 16;
+    float* planes = partials + (size_t)blockIdx.y * NS * M * npad + strip * 16 + 4 * kq;
 #pragma unroll
     for (int g = 0; g < NS; g++)
 #pragma unroll
-      for (int mt = 0; mt < MT; mt++) mine[(g * MT + mt) * 64] = acc[g][mt];
+      for (int mt = 0; mt < MT; mt++)
+        if (mt * 16 + r < M) *(f32x4*)(planes + ((size_t)g * M + mt * 16 + r) * npad) = acc[g][mt];
     return;
   }
   if (strip_ok) mid_store<MT, GATED>(acc, C, ldc, c_is_f32, M, N, strip, lane, epi, cap);
 }
 
-// Second half of a product whose K was split over blocks: the partial sums of a column block,
-// added in the order of the ranges, then the epilogue.  Same lanes, same values per lane as in
-// the product kernel.
-template <int MT, bool GATED>
-__global__ __launch_bounds__(256) void gemm_mid_join_kernel(const f32x4* __restrict__ partials, int ksplit,
-                                                            void* __restrict__ C, int ldc, int c_is_f32,
-                                                            int M, int N, int epi, float cap) {
+// Second half of a mid product whose K was split over blocks: `ksplit`
+// ranges of one ([M, npad] floats) or, GATED, two planes each; a thread adds four neighbouring
+// columns of a row in the order of the ranges and applies the epilogue.  A reader that adds the
+// planes up itself in the same order (zk_norm_add_norm) makes this launch unnecessary.
+template <bool GATED>
+__global__ __launch_bounds__(256) void gemm_join_kernel(const float* __restrict__ partials, int ksplit,
+                                                        void* __restrict__ C, int ldc, int c_is_f32, int M,
+                                                        int N, int npad, int epi, float cap) {
   constexpr int NS = GATED ? 2 : 1;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int strip = blockIdx.x * 4 + wave;
-  if (strip >= (N + 15) / 16) return;
-  const f32x4* all = partials + (((size_t)blockIdx.x * ksplit) * 4 + wave) * (NS * MT * 64) + lane;
-  f32x4 acc[NS][MT];
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const int m = (int)(idx / (npad / 4)), n = (int)(idx % (npad / 4)) * 4;
+  if (m >= M) return;
+  const size_t plane = (size_t)M * npad;
+  const float* at = partials + (size_t)m * npad + n;
+  f32x4 x = *(const f32x4*)at, y = x;
+  if (GATED) y = *(const f32x4*)(at + plane);
+  for (int p = 1; p < ksplit; p++) {
+    x += *(const f32x4*)(at + (size_t)p * NS * plane);
+    if (GATED) y += *(const f32x4*)(at + ((size_t)p * NS + 1) * plane);
+  }
 #pragma unroll
-  for (int g = 0; g < NS; g++)
-#pragma unroll
-    for (int mt = 0; mt < MT; mt++) acc[g][mt] = all[(g * MT + mt) * 64];
-  for (int p = 1; p < ksplit; p++)
-#pragma unroll
-    for (int g = 0; g < NS; g++)
-#pragma unroll
-      for (int mt = 0; mt < MT; mt++) acc[g][mt] += all[((size_t)p * 4 * NS * MT + g * MT + mt) * 64];
-  mid_store<MT, GATED>(acc, C, ldc, c_is_f32, M, N, strip, lane, epi, cap);
+  for (int i = 0; i < 4; i++) {
+    if (n + i >= N) continue;
+    float v = x[i];
+    if (GATED) v = epi_gate(v, y[i], epi);
+    else if (epi == EPI_SOFTCAP) v = cap * tanhf(v / cap);
+    if (c_is_f32) ((float*)C)[(size_t)m * ldc + n + i] = v;
+    else ((__bf16*)C)[(size_t)m * ldc + n + i] = (__bf16)v;
+  }
 }
 
 template <bool GATED>
 static int launch_mid(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M, int N,
-                      int K, int epi, float cap, void* ws, size_t ws_bytes, hipStream_t s) {
+                      int K, int epi, float cap, void* ws, size_t ws_bytes, int* parts, hipStream_t s) {
   const int mt = (M + 15) / 16;
+  const int npad = (N + 15) / 16 * 16;
   const int cblocks = ((N + 15) / 16 + 3) / 4;
   // split K until every CU has a block, a range no shorter than a chunk; more ranges than that
   // cost more in partial sums than they gain (measured at N = 2304 and 4096, M = 32 and 64)
   int ksplit = 256 / cblocks;
   if (ksplit > K / 32 / GM_STEPS) ksplit = K / 32 / GM_STEPS;
   if (ksplit < 1) ksplit = 1;
-  const size_t per_range = (size_t)4 * (GATED ? 2 : 1) * mt * 64 * sizeof(f32x4);
+  const size_t per_range = (size_t)(GATED ? 2 : 1) * M * npad * sizeof(float);
   if (ws == nullptr || (uintptr_t)ws % 16 != 0) ksplit = 1;
-  while (ksplit > 1 && (size_t)cblocks * ksplit * per_range > ws_bytes) ksplit--;
-  f32x4* partials = (f32x4*)ws;
+  while (ksplit > 1 && ksplit * per_range > ws_bytes) ksplit--;
+  float* partials = (float*)ws;
   dim3 grid(cblocks, ksplit);
 #define ZK_MID(MT_)                                                                                   \
   gemm_mid_kernel<MT_, GATED><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, \
-                                                   M, N, K, epi, cap, partials, ksplit);                \
-  if (ksplit > 1)                                                                                     \
-    gemm_mid_join_kernel<MT_, GATED><<<cblocks, 256, 0, s>>>(partials, ksplit, C, ldc, c_is_f32, M, N, epi, cap)
+                                                   M, N, K, epi, cap, partials, ksplit)
   if (mt == 2) { ZK_MID(2); }
   else if (mt == 3) { ZK_MID(3); }
   else { ZK_MID(4); }
 #undef ZK_MID
+  if (ksplit > 1) {
+    if (parts && joinable_by_reader(N, ldc, c_is_f32, epi)) {
+      *parts = ksplit;
+      return zk_launch_status("zk_gemm_bf16 (mid)");
+    }
+    const size_t quads = (size_t)M * (npad / 4);
+    gemm_join_kernel<GATED><<<(unsigned)((quads + 255) / 256), 256, 0, s>>>(partials, ksplit, C, ldc, c_is_f32, M, N,
+                                                                          npad, epi, cap);
+  }
   return zk_launch_status("zk_gemm_bf16 (mid)");
 }
 
@@ -836,13 +863,16 @@ extern "C" int zk_strip_layout(const void* src, void* dst, int N, int K, void* s
 // epilogues W is [2N, K] (gate rows, then up rows) and C is [M, N].
 // w_strip: W is in strip layout (zk_strip_layout), which needs K % 32 == 0 and, for the
 // gated epilogues, N % 16 == 0.
-// The workspace may be null; then K is never split over blocks.  It holds nothing between
-// launches and serves one launch at a time.
+// The workspace may be null; then K is never split over blocks.  It serves one launch at a time.
+// parts (may be null): a caller whose next kernel can add partial sums up itself passes a place
+// for their number.  0 comes back when the result is in C as usual; P > 0 when C was not
+// written and the workspace starts with P planes of [M, N] floats, to be added in order and
+// rounded to 16 bits (zk_norm_add_norm reads them so), before the next product overwrites them.
 extern "C" size_t zk_gemm_bf16_workspace() { return (size_t)32 << 20; }
 
 extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
                             int M, int N, int K, int epi, float cap, int w_strip, void* ws,
-                            size_t ws_bytes, void* stream) {
+                            size_t ws_bytes, int* parts, void* stream) {
   ZK_REQUIRE(M >= 0 && N > 0 && K > 0, "zk_gemm_bf16: bad sizes");
   ZK_REQUIRE(K % 8 == 0 && lda % 8 == 0, "zk_gemm_bf16: K and lda must be multiples of 8");
   ZK_REQUIRE(lda >= K && ldc >= N, "zk_gemm_bf16: leading dimensions too small");
@@ -851,11 +881,12 @@ extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int 
   ZK_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "zk_gemm_bf16: operands must be 16-byte aligned");
   const bool gated = epi >= EPI_GELU_TANH;
   ZK_REQUIRE(!w_strip || (K % 32 == 0 && (!gated || N % 16 == 0)), "zk_gemm_bf16: strip layout needs K % 32 == 0 (and N % 16 == 0 when gated)");
+  if (parts) *parts = 0;
   if (M == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (M > 16 && M <= 64 && w_strip) {
-    return gated ? launch_mid<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, ws, ws_bytes, s)
-                 : launch_mid<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, ws, ws_bytes, s);
+    return gated ? launch_mid<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, ws, ws_bytes, parts, s)
+                 : launch_mid<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, ws, ws_bytes, parts, s);
   }
   if (M <= 64) {
     return gated ? launch_skinny<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s)

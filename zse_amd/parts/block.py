@@ -46,14 +46,19 @@ class Block(Part):
             out = ctx.alloc((T, H))
         ps = post.spec if post is not None else None
         ns = nxt.spec if (nxt is not None and fused_next) else None
+        parts = sub.shape[0] if sub.layout == "parts" else 0     # partial sums of a product that split K
         ctx.k.zk_norm_add_norm(
-            sub.ptr, post.weight.ptr if post is not None else None, ps.eps if ps else 0.0,
+            sub.ptr, parts, post.weight.ptr if post is not None else None, ps.eps if ps else 0.0,
             int(ps.unit_offset) if ps else 0, h.ptr,
             nxt.weight.ptr if ns else None, ns.eps if ns else 0.0, int(ns.unit_offset) if ns else 0,
             out.ptr if out is not None else None, T, H, ctx.stream)
         if nxt is not None and not fused_next:
             out = nxt.forward(ctx, h)
         return out
+
+    @staticmethod
+    def _joins_sums(post) -> bool:
+        return post is None or isinstance(post, RMSNorm)
 
     def entry_norm(self):
         """The norm this block applies to the stream first; the block before may apply it
@@ -67,9 +72,14 @@ class Block(Part):
         residual sum), in ``x_out`` if given."""
         n = self.norms
         x = x_in if x_in is not None else n["pre_mixer"].forward(ctx, h)
+        # the joining kernel adds up the partial sums of a part's last product itself
+        ctx.sums_welcome = self._joins_sums(n.get("post_mixer"))
         a = self.mixer.forward(ctx, x, cache)
+        ctx.sums_welcome = False
         x = self._join(ctx, a, n.get("post_mixer"), h, n["pre_ffn"])
+        ctx.sums_welcome = self._joins_sums(n.get("post_ffn"))
         m = self.ffn.forward(ctx, x)
+        ctx.sums_welcome = False
         if not isinstance(next_norm, RMSNorm):
             next_norm = None         # a norm the closing kernel does not know: the next block applies it
         return self._join(ctx, m, n.get("post_ffn"), h, next_norm, x_out)

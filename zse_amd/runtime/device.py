@@ -143,7 +143,7 @@ _VP, _I, _F, _SZ, _U64 = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint64
 KERNEL_SIGNATURES = {
     "zk_embed": [_VP, _VP, _VP, _F, _I, _I, _I, _I, _VP],
     "zk_rmsnorm": [_VP, _I, _VP, _VP, _VP, _F, _I, _I, _I, _VP],
-    "zk_norm_add_norm": [_VP, _VP, _F, _I, _VP, _VP, _F, _I, _VP, _I, _I, _VP],
+    "zk_norm_add_norm": [_VP, _I, _VP, _F, _I, _VP, _VP, _F, _I, _VP, _I, _I, _VP],
     "zk_gated_act": [_VP, _VP, _I, _I, _I, _VP],
     "zk_softcap": [_VP, _SZ, _F, _VP],
     "zk_rope_cache_write": [_VP, _VP, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
@@ -158,7 +158,7 @@ KERNEL_SIGNATURES = {
 }
 # present only in the bf16 library
 BF16_KERNEL_SIGNATURES = {
-    "zk_gemm_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, C.c_size_t, _VP],
+    "zk_gemm_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, C.c_size_t, C.POINTER(C.c_int), _VP],
     "zk_strip_layout": [_VP, _VP, _I, _I, _VP],
     "zk_qkv_rope_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "zk_attention_bf16": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
