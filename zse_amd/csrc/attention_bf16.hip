@@ -90,7 +90,9 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
   // Decoded tokens: a wave owns one chunk of keys.
   int gi = 0, phase = wave, nphase = 4, first_wave = 0;        // group, and the wave's place among its waves
   int na_block = 4;                                            // waves of the block's first group
-  if (!SPLIT && !PAIR) gi = blockIdx.x;
+  // single groups: the last group of a portion sees the most keys and goes first, so that the
+  // blocks still running at the end are the short ones
+  if (!SPLIT && !PAIR) gi = (n + p.tpw - 1) / p.tpw - 1 - (int)blockIdx.x;
   if (PAIR) {
     const int groups = (n + p.tpw - 1) / p.tpw;
     if ((int)blockIdx.x >= (groups + 1) / 2) return;           // the whole block is past the portion
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
   }
   const int chunk = SPLIT ? blockIdx.x * 4 + wave : 0;
   const int t0 = gi * p.tpw;
-  if (!PAIR && t0 >= n) return;
+  if (!PAIR && (gi < 0 || t0 >= n)) return;
   const int g = p.nh / p.nkv;
   const int tok = lr / g, hq = lr - tok * g;
   const int ntok = min(p.tpw, n - t0);
@@ -149,33 +151,56 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
 #pragma unroll
     for (int e = 0; e < 16; e++) o[dt][e] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
+  // where the lane's channels dt * 32 + lr lie in a (page, kv head) block of the transposed V cache
+  int vrow[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++) vrow[dt] = min(dt * 32 + lr, hd - 1) << bsh;
+  const bool capped = p.softcap > 0.f;
+  // keys every row of the group sees (none beyond the first row's position, none before the
+  // last row's window; no range at all unless every lane holds a row): tiles inside this range
+  // need no mask
+  const int all_hi = ntok * g == 32 ? pos_lo : -1;
+  const int all_lo = p.window > 0 ? max(0, pos_hi - p.window + 1) : 0;
 
-  for (int key0 = (key_lo / 32) * 32 + (SPLIT ? 0 : phase * 32); key0 <= key_hi; key0 += SPLIT ? 32 : 32 * nphase) {
+  // The pages of a tile are looked up a tile ahead as well, so that no load waits for a table
+  // entry: the lane's key row, and the four places its V pieces come from.
+  struct TilePages { int k, va[2], vb[2]; };
+  auto look_up = [&](int key0, TilePages& pg) {
+    pg.k = table[min(key0 + lr, key_hi) >> bsh];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      pg.va[h] = table[min(key0 + h * 16 + 4 * lk, key_hi & ~3) >> bsh];
+      pg.vb[h] = table[min(key0 + h * 16 + 8 + 4 * lk, key_hi & ~3) >> bsh];
+    }
+  };
+  auto load_k = [&](int key0, int page, bf16x8 (&kf)[HD16]) {
+    const int kk = min(key0 + lr, key_hi);
+    const __bf16* kr = p.kcache + ((((size_t)max(page, 0) * nkv + kvh) << bsh) + (kk & bmask)) * hd + lk * 8;
+#pragma unroll
+    for (int ks = 0; ks < HD16; ks++) kf[ks] = *(const bf16x8*)(kr + ks * 16);
+  };
+  auto tile = [&](int key0, const TilePages& pg, int knext, TilePages& pn) {
+    bf16x8 kf[HD16];
+    load_k(key0, pg.k, kf);
+    look_up(knext, pn);
     // ---- S^T = K Q^T
     f32x16 s;
 #pragma unroll
     for (int e = 0; e < 16; e++) s[e] = 0.f;
-    {
-      const int kk = min(key0 + lr, key_hi);
-      const int page = max(table[kk >> bsh], 0);
-      const __bf16* kr = p.kcache + ((((size_t)page * nkv + kvh) << bsh) + (kk & bmask)) * hd + lk * 8;
-      bf16x8 kf[HD16];
 #pragma unroll
-      for (int ks = 0; ks < HD16; ks++) kf[ks] = *(const bf16x8*)(kr + ks * 16);
-#pragma unroll
-      for (int ks = 0; ks < HD16; ks++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], s, 0, 0, 0);
-    }
+    for (int ks = 0; ks < HD16; ks++) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], s, 0, 0, 0);
     // ---- V^T pieces for this tile (issued early; used after the softmax)
     bf16x8 vf[DT][2];
 #pragma unroll
     for (int h = 0; h < 2; h++) {
       const int ka = min(key0 + h * 16 + 4 * lk, key_hi & ~3), kb = min(key0 + h * 16 + 8 + 4 * lk, key_hi & ~3);
-      const int pa = max(table[ka >> bsh], 0), pb = max(table[kb >> bsh], 0);
+      const int pa = max(pg.va[h], 0), pb = max(pg.vb[h], 0);
+      const __bf16* vpa = p.vcache + ((((size_t)pa * nkv + kvh) * hd) << bsh) + (ka & bmask);
+      const __bf16* vpb = p.vcache + ((((size_t)pb * nkv + kvh) * hd) << bsh) + (kb & bmask);
 #pragma unroll
       for (int dt = 0; dt < DT; dt++) {
-        const int d = min(dt * 32 + lr, hd - 1);
-        const bf16x4 va = *(const bf16x4*)(p.vcache + (((((size_t)pa * nkv + kvh) * hd + d)) << bsh) + (ka & bmask));
-        const bf16x4 vb = *(const bf16x4*)(p.vcache + (((((size_t)pb * nkv + kvh) * hd + d)) << bsh) + (kb & bmask));
+        const bf16x4 va = *(const bf16x4*)(vpa + vrow[dt]);
+        const bf16x4 vb = *(const bf16x4*)(vpb + vrow[dt]);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           vf[dt][h][e] = va[e];
@@ -185,17 +210,28 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
     }
     // ---- scale, cap, mask, running softmax (one query row per lane)
     float mt = -INFINITY;
+    if (capped) {
 #pragma unroll
-    for (int j = 0; j < 4; j++)
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int key = key0 + 8 * j + 4 * lk + i;
-        float v = score_log2(p, s[4 * j + i]);
-        const bool ok = row_ok && key >= row_lo && key <= pos && key >= key_lo && key <= key_hi;
-        v = ok ? v : -INFINITY;
-        s[4 * j + i] = v;
-        mt = fmaxf(mt, v);
+      for (int e = 0; e < 16; e++) {
+        const float ex = __builtin_amdgcn_exp2f(p.k2 * s[e]);
+        s[e] = p.c2 * (1.f - 2.f * __builtin_amdgcn_rcpf(ex + 1.f));
       }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 16; e++) s[e] *= p.k1;
+    }
+    if (key0 < all_lo || key0 + 31 > all_hi || key0 < key_lo || key0 + 31 > key_hi) {
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int key = key0 + 8 * j + 4 * lk + i;
+          const bool ok = row_ok && key >= row_lo && key <= pos && key >= key_lo && key <= key_hi;
+          s[4 * j + i] = ok ? s[4 * j + i] : -INFINITY;
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 16; e++) mt = fmaxf(mt, s[e]);
     mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
     const float m_new = mt > m_run + 8.f ? mt : m_run;      // the reference follows the maximum lazily
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
@@ -216,17 +252,38 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
     for (int h = 0; h < 2; h++)
 #pragma unroll
       for (int e = 0; e < 8; e++) pb[h][e] = (__bf16)s[8 * h + e];
-    // ---- O^T = corr * O^T + V^T P^T
-    if (__any(moved)) {
+    // ---- O^T = corr * O^T + V^T P^T  (the maximum rarely rises by the threshold after a
+    // row's first tiles; said so, the compiler keeps the accumulators where the products
+    // want them instead of moving all of them on every tile)
+    if (__builtin_expect(__any(moved), 0)) {
+      // in the accumulation registers, where the products keep them: written so, the compiler
+      // does not copy all of them to ordinary registers on every tile for this rare path
 #pragma unroll
       for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-        for (int e = 0; e < 16; e++) o[dt][e] *= corr;
+        for (int e = 0; e < 16; e++) {
+          float t;
+          asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
+                       : "+a"(o[dt][e]), "=&v"(t)
+                       : "v"(corr));
+        }
     }
 #pragma unroll
     for (int dt = 0; dt < DT; dt++) {
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][0], pb[0], o[dt], 0, 0, 0);
       o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][1], pb[1], o[dt], 0, 0, 0);
+    }
+  
+  };
+  {
+    const int kstep = SPLIT ? 32 : 32 * nphase;
+    int key0 = (key_lo / 32) * 32 + (SPLIT ? 0 : phase * 32);
+    TilePages p0, p1;
+    if (key0 <= key_hi) look_up(key0, p0);
+    for (; key0 <= key_hi; key0 += 2 * kstep) {
+      tile(key0, p0, key0 + kstep, p1);
+      if (key0 + kstep > key_hi) break;
+      tile(key0 + kstep, p1, key0 + 2 * kstep, p0);
     }
   }
   if (SPLIT) {

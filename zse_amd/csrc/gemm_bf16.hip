@@ -1,14 +1,16 @@
 // bfloat16 matrix products on the matrix cores (MFMA), float accumulation:
 //   C[M,N] = A[M,K] * W[N,K]^T        (weights [out, in], both operands K-contiguous)
 //
-// Two kernels, chosen by M:
-//  * skinny (M <= 64, decode): the weight matrix is streamed once from HBM.  A
-//    block owns a strip of 16 weight rows; its four waves split K and each feeds
-//    16x16x32 MFMAs straight from global memory: a lane's 16-byte load is exactly
-//    its MFMA operand (row = lane % 16, eight k values at 8 * (lane / 16)), so no
-//    LDS staging is needed.  Partial sums of the four waves meet in LDS.
-//  * tile (M > 64, prefill): 256x128x64 or 128x128x64 block tiles staged through LDS, four waves
-//    of 64 lanes, each a 128x64 or 64x64 corner built from 32x32x16 MFMAs.
+// Three kernels, chosen by M:
+//  * skinny (M <= 16, or weights not in strip layout up to 64): the weight matrix is streamed
+//    once from HBM.  A block owns a strip of 16 weight rows; its waves split K and each feeds
+//    16x16x32 MFMAs straight from global memory: a lane's 16-byte load is exactly its MFMA
+//    operand (row = lane % 16, eight k values at 8 * (lane / 16)), so no LDS staging is
+//    needed.  Partial sums of the waves meet in LDS.
+//  * mid (17 <= M <= 64, strip layout): four strips a block, the activations of a k chunk
+//    shared through LDS, K split over blocks when N alone gives too few of them.
+//  * tile (M > 64, prefill): 128x256x64 (eight waves) or 128x128x64 (four) block tiles staged
+//    through LDS, each wave a 64x64 corner built from 32x32x16 MFMAs.
 // Epilogues: plain store (bf16 or float), soft cap on float output (LM head), and
 // the gated activation act(gate) * up over a [2I, K] weight whose first I rows are
 // the gate (the feed-forward's first product; the [T, 2I] intermediate never
