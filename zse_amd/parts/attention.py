@@ -103,7 +103,7 @@ class PagedAttention(Part):
                                  g.max_blocks, ctx.req_of_token, ctx.positions, o.ptr, T, nh, nkv,
                                  hd, g.page_size, s.scale, cap, win, 1 if cache.v_transposed else 0,
                                  ctx.stream)
-        return linear(ctx, o, self.w_o, ctx.alloc((T, s.hidden_size)), last=True)
+        return linear(ctx, o, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)
 
 
 register_part("mixer", "attention", PagedAttention)

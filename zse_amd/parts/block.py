@@ -73,13 +73,12 @@ class Block(Part):
         n = self.norms
         x = x_in if x_in is not None else n["pre_mixer"].forward(ctx, h)
         # the joining kernel adds up the partial sums of a part's last product itself
-        ctx.sums_welcome = self._joins_sums(n.get("post_mixer"))
+        ctx.sums_welcome = self.mixer if self._joins_sums(n.get("post_mixer")) else None
         a = self.mixer.forward(ctx, x, cache)
-        ctx.sums_welcome = False
         x = self._join(ctx, a, n.get("post_mixer"), h, n["pre_ffn"])
-        ctx.sums_welcome = self._joins_sums(n.get("post_ffn"))
+        ctx.sums_welcome = self.ffn if self._joins_sums(n.get("post_ffn")) else None
         m = self.ffn.forward(ctx, x)
-        ctx.sums_welcome = False
+        ctx.sums_welcome = None
         if not isinstance(next_norm, RMSNorm):
             next_norm = None         # a norm the closing kernel does not know: the next block applies it
         return self._join(ctx, m, n.get("post_ffn"), h, next_norm, x_out)

@@ -43,11 +43,11 @@ class GatedMLP(Part):
         T, I = x.shape[0], s.intermediate_size
         if tuned_gemm(ctx, s.hidden_size):
             a = linear(ctx, x, self.w_gu, ctx.alloc((T, I)), epilogue=s.activation)
-            return linear(ctx, a, self.w_down, ctx.alloc((T, s.hidden_size)), last=True)
+            return linear(ctx, a, self.w_down, ctx.alloc((T, s.hidden_size)), last_of=self)
         gu = linear(ctx, x, self.w_gu, ctx.alloc((T, 2 * I)))
         a = ctx.alloc((T, I))
         ctx.k.zk_gated_act(gu.ptr, a.ptr, T, I, ACTIVATION_CODES[s.activation], ctx.stream)
-        return linear(ctx, a, self.w_down, ctx.alloc((T, s.hidden_size)), last=True)
+        return linear(ctx, a, self.w_down, ctx.alloc((T, s.hidden_size)), last_of=self)
 
 
 register_part("ffn", "gated_mlp", GatedMLP)
