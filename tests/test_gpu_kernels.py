@@ -611,7 +611,7 @@ def test_argmax_and_sampling(rt):
     z[3, 5] = np.nan
     Z = rt.upload(z)
     ids = rt.empty((rows,), "int32")
-    scratch = rt.empty((rows * 128,), "float32")
+    scratch = rt.empty((rows * 64 * 5,), "float32")
     k.zk_argmax(Z.ptr, ids.ptr, rows, V, scratch.ptr, rt.stream)
     got = rt.download(ids)
     want = [int(np.nanargmax(r)) for r in z]
@@ -625,14 +625,41 @@ def test_argmax_and_sampling(rt):
     z = rng.normal(size=(rows, 1000)).astype(np.float32) * 2
     temps = np.array([0.8, 1.0, 0.3, 2.0, 1.0], np.float32)
     us = np.array([0.0, 0.999999, 0.5, 0.25, 0.75])
-    k.zk_sample(ptr(rt.upload(z)), ptr(rt.upload(temps)), ptr(rt.upload(us)), None, ids.ptr, rows, 1000, rt.stream)
+    k.zk_sample(ptr(rt.upload(z)), ptr(rt.upload(temps)), ptr(rt.upload(us)), None, None, ids.ptr, rows, 1000, scratch.ptr, rt.stream)
     assert list(rt.download(ids)) == [P.sample(z[i], us[i], temperature=float(temps[i])) for i in range(rows)]
     # the frequencies follow softmax(z / T)
     z1 = np.array([[2.0, 1.0, 0.0, -1.0]], np.float32).repeat(4000, 0)
     from zse_amd.sampling import uniform
     u = np.array([uniform(3, i) for i in range(4000)])
     out = rt.empty((4000,), "int32")
-    k.zk_sample(ptr(rt.upload(z1)), ptr(rt.upload(np.full(4000, 0.7, np.float32))), ptr(rt.upload(u)), None, out.ptr,
-                4000, 4, rt.stream)
+    k.zk_sample(ptr(rt.upload(z1)), ptr(rt.upload(np.full(4000, 0.7, np.float32))), ptr(rt.upload(u)), None, None, out.ptr,
+                4000, 4, ptr(rt.empty((4000 * 64 * 5,), "float32")), rt.stream)
     freq = np.bincount(rt.download(out), minlength=4) / 4000.0
     assert np.abs(freq - P.softmax(z1[0] / 0.7)).max() < 0.03
+
+
+@pytest.mark.parametrize("V,ties", [(5003, False), (5003, True), (256000, False), (37, True)])
+def test_top_k_top_p_and_penalty_on_the_device(rt, V, ties):
+    """Every combination goes through the device sampler and picks what the host implementation
+    (float64, sorting) picks for the same uniform number; with logits on a coarse grid many are
+    equal, also at the cut-offs, where top-k keeps all of them and top-p the first few."""
+    from zse_amd.sampling import DeviceSampler, SamplingParams, sample_host, uniform
+    rng = np.random.default_rng(V + ties)
+    combos = [dict(top_k=k_, top_p=p_, temperature=t_, repetition_penalty=r_)
+              for k_ in (0, 1, 5, 50, V + 10) for p_ in (1.0, 0.9, 0.5, 0.02) for t_, r_ in ((0.7, 1.0), (1.3, 1.5))]
+    combos += [dict(temperature=0.0, repetition_penalty=3.0), dict(temperature=0.0, top_k=3)]
+    n = len(combos)
+    z = (rng.normal(size=(n, V)) * 3).astype(np.float32)
+    if ties:
+        z = (np.round(z * 2) / 2).astype(np.float32)
+    sampler = DeviceSampler(rt, rt.kernels("float32"), n)
+    for trial in range(3):
+        rows = []
+        for i, c in enumerate(combos):
+            order = np.argsort(-z[i])
+            past = set(order[:3].tolist()) | set(rng.integers(0, V, 5).tolist())
+            rows.append({"params": SamplingParams(**c), "u": uniform(trial * 1000 + i, 7) if trial else (0.0, 0.999999)[i % 2],
+                         "past": past})
+        got = sampler.sample(rt.upload(z), rows)                 # the penalty changes the logits in place: a fresh copy
+        want = [sample_host(z[i], r["params"], r["u"], r["past"]) for i, r in enumerate(rows)]
+        assert got == want, [(i, combos[i], g, w) for i, (g, w) in enumerate(zip(got, want)) if g != w]

@@ -57,5 +57,5 @@ def test_params_validate():
         with pytest.raises(ValueError):
             SamplingParams(**bad)
     assert SamplingParams(temperature=0).greedy and SamplingParams(temperature=1e-7).greedy
-    assert SamplingParams(temperature=0.8).on_device and not SamplingParams(top_k=5).on_device
-    assert SamplingParams(temperature=0, top_k=5).on_device
+    assert SamplingParams(temperature=0.8).plain and not SamplingParams(top_k=5).plain
+    assert SamplingParams(temperature=0, top_k=5).plain and not SamplingParams(temperature=0, repetition_penalty=1.2).plain

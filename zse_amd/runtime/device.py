@@ -154,7 +154,9 @@ KERNEL_SIGNATURES = {
     "zk_attention_plain": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _F,
                            _I, _I, _VP],
     "zk_argmax": [_VP, _VP, _I, _I, _VP, _VP],
-    "zk_sample": [_VP, _VP, _VP, _VP, _VP, _I, _I, _VP],
+    "zk_sample": [_VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP],
+    "zk_sample_cutoff": [_VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP],
+    "zk_penalize": [_VP, _I, _VP, _VP, _VP, _I, _VP],
 }
 # present only in the bf16 library
 BF16_KERNEL_SIGNATURES = {

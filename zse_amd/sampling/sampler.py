@@ -11,9 +11,11 @@ given, and the uniform number is a pure function of (seed, index of the
 output token) instead of coming from one shared generator (:30-31), so a
 request samples the same tokens whatever else is in the batch.
 
-Greedy and plain temperature sampling run on the device
-(csrc/sampling.hip); rows that use top-k, top-p or a penalty are brought to the
-host, where the reference samples everything (:10-11).
+All of it runs on the device (csrc/sampling.hip): the penalty as a small
+kernel over the (row, token) pairs, top-k and top-p as a cut-off value and a
+number of its ties per row, then the argmax or the inverse CDF.  The host
+implementation below is the same arithmetic in float64 and what the device is
+tested against; the reference samples everything on the host (:10-11).
 """
 from __future__ import annotations
 
@@ -52,8 +54,9 @@ class SamplingParams:
         return self.temperature <= 0 or self.temperature < 1e-6
 
     @property
-    def on_device(self) -> bool:
-        """True when the device kernels cover this request's sampling."""
+    def plain(self) -> bool:
+        """Greedy or temperature alone: nothing but the logits and a uniform number is needed,
+        so runs of steps can be enqueued without the host in between."""
         return self.repetition_penalty == 1.0 and (self.greedy or (self.top_k == 0 and self.top_p >= 1.0))
 
 
@@ -76,11 +79,15 @@ def fresh_seed() -> int:
 
 # ---------------------------------------------------------------- host sampling
 
-def apply_repetition_penalty(z: np.ndarray, past: Iterable[int], penalty: float) -> np.ndarray:
+def penalty_scales(past: Iterable[int], penalty: float) -> Dict[int, float]:
+    """Token id -> what its logit is divided (if positive) or multiplied by."""
     counts: Dict[int, int] = past if isinstance(past, dict) else {int(t): 1 for t in past}
-    for tid, cnt in counts.items():
+    return {int(t): (penalty ** (1.0 + math.log2(c)) if c > 1 else penalty) for t, c in counts.items()}
+
+
+def apply_repetition_penalty(z: np.ndarray, past: Iterable[int], penalty: float) -> np.ndarray:
+    for tid, s in penalty_scales(past, penalty).items():
         if 0 <= tid < len(z):
-            s = penalty ** (1.0 + math.log2(cnt)) if cnt > 1 else penalty
             z[tid] = z[tid] / s if z[tid] > 0 else z[tid] * s
     return z
 
@@ -134,15 +141,20 @@ class DeviceSampler:
         self.ids2 = rt.empty((max_rows,), I32)
         self.temp = rt.empty((max_rows,), F32)
         self.u = rt.empty((max_rows,), F64)
-        self.scratch = rt.empty((max_rows * 128,), F32)     # slices of the two-stage argmax
+        self.scratch = rt.empty((max_rows * 64 * 5,), F32)  # per row 64 slices: a double, a float, an int
+        self.top_k = rt.empty((max_rows,), I32)
+        self.top_p = rt.empty((max_rows,), F32)
+        self.keep_from = rt.empty((max_rows,), F32)
+        self.keep_ties = rt.empty((max_rows,), I32)
+        self._pen = None                                    # (rows, tokens, scales) on the device, grown on demand
 
     # ---- a run of steps without waiting for the host in between
     RING = 16       # results that may be on their way to the host at a time
 
     def can_defer(self, rows: Sequence[dict]) -> bool:
-        """True when ``sample_deferred`` serves these rows: all on the device, all greedy or
-        all drawn with a temperature."""
-        if not rows or len(rows) > self.max_rows or not all(r["params"].on_device for r in rows):
+        """True when ``sample_deferred`` serves these rows: nothing but greedy or temperature,
+        and all of one kind."""
+        if not rows or len(rows) > self.max_rows or not all(r["params"].plain for r in rows):
             return False
         kinds = {bool(r["params"].greedy) for r in rows}
         return len(kinds) == 1
@@ -172,8 +184,8 @@ class DeviceSampler:
             k.zk_argmax(logits.ptr, self.ids.ptr, n, V, self.scratch.ptr, rt.stream)
             dev = self.ids
         else:
-            k.zk_sample(logits.ptr, self.temp.ptr, self._run_u.ptr + step_in_run * n * 8, None, self.ids2.ptr,
-                        n, V, rt.stream)
+            k.zk_sample(logits.ptr, self.temp.ptr, self._run_u.ptr + step_in_run * n * 8, None, None,
+                        self.ids2.ptr, n, V, self.scratch.ptr, rt.stream)
             dev = self.ids2
         if getattr(self, "_ring", None) is None:
             self._ring = [(rt.pinned(self.max_rows * 4), rt.event()) for _ in range(self.RING)]
@@ -193,26 +205,42 @@ class DeviceSampler:
         if n > self.max_rows:
             raise ValueError(f"{n} rows to sample, room for {self.max_rows}")
         rt, k = self.rt, self.k
-        need_greedy = any(r["params"].on_device and r["params"].greedy for r in rows)
-        need_temp = any(r["params"].on_device and not r["params"].greedy for r in rows)
-        need_host = [i for i, r in enumerate(rows) if not r["params"].on_device]
-        out: List[Optional[int]] = [None] * n
-        if need_greedy:
+        # the penalty first, in place: what follows sees the changed logits, greedy rows too
+        pen = [(i, t, sc) for i, r in enumerate(rows) if r["params"].repetition_penalty != 1.0 and r.get("past")
+               for t, sc in penalty_scales(r["past"], r["params"].repetition_penalty).items() if 0 <= t < V]
+        if pen:
+            self._penalize(logits, V, pen)
+        greedy = [bool(r["params"].greedy) for r in rows]
+        if any(greedy):
             k.zk_argmax(logits.ptr, self.ids.ptr, n, V, self.scratch.ptr, rt.stream)
-        if need_temp:
-            t = np.array([r["params"].temperature if not r["params"].greedy else 1.0 for r in rows],
-                         dtype=np.float32)
+        if not all(greedy):
+            t = np.array([1.0 if g else r["params"].temperature for r, g in zip(rows, greedy)], dtype=np.float32)
             u = np.array([r["u"] for r in rows], dtype=np.float64)
             rt.copy_h2d(self.temp.ptr, t)
             rt.copy_h2d(self.u.ptr, u)
-            k.zk_sample(logits.ptr, self.temp.ptr, self.u.ptr, None, self.ids2.ptr, n, V, rt.stream)
-        g = rt.download(self.ids.rows(0, n)) if need_greedy else None
-        s = rt.download(self.ids2.rows(0, n)) if need_temp else None
-        for i, r in enumerate(rows):
-            p = r["params"]
-            if p.on_device:
-                out[i] = int(g[i]) if p.greedy else int(s[i])
-        for i in need_host:
-            row = rt.download(logits.rows(i, i + 1))[0]
-            out[i] = sample_host(row, rows[i]["params"], rows[i]["u"], rows[i].get("past", ()))
-        return out
+            cut = any(not g and not r["params"].plain and (r["params"].top_k > 0 or r["params"].top_p < 1.0)
+                      for r, g in zip(rows, greedy))
+            if cut:
+                rt.copy_h2d(self.top_k.ptr, np.array([0 if g else r["params"].top_k for r, g in zip(rows, greedy)],
+                                                     dtype=np.int32))
+                rt.copy_h2d(self.top_p.ptr, np.array([1.0 if g else r["params"].top_p for r, g in zip(rows, greedy)],
+                                                     dtype=np.float32))
+                k.zk_sample_cutoff(logits.ptr, self.temp.ptr, self.top_k.ptr, self.top_p.ptr, self.keep_from.ptr,
+                                   self.keep_ties.ptr, n, V, rt.stream)
+            k.zk_sample(logits.ptr, self.temp.ptr, self.u.ptr, self.keep_from.ptr if cut else None,
+                        self.keep_ties.ptr if cut else None, self.ids2.ptr, n, V, self.scratch.ptr, rt.stream)
+        g = rt.download(self.ids.rows(0, n)) if any(greedy) else None
+        s = rt.download(self.ids2.rows(0, n)) if not all(greedy) else None
+        return [int(g[i]) if greedy[i] else int(s[i]) for i in range(n)]
+
+    def _penalize(self, logits, V: int, pen) -> None:
+        from ..runtime.device import F32, I32
+        m = len(pen)
+        if self._pen is None or self._pen[0].shape[0] < m:
+            room = max(1024, 2 * m)
+            self._pen = (self.rt.empty((room,), I32), self.rt.empty((room,), I32), self.rt.empty((room,), F32))
+        rows_d, toks_d, scales_d = self._pen
+        self.rt.copy_h2d(rows_d.ptr, np.array([p[0] for p in pen], dtype=np.int32))
+        self.rt.copy_h2d(toks_d.ptr, np.array([p[1] for p in pen], dtype=np.int32))
+        self.rt.copy_h2d(scales_d.ptr, np.array([p[2] for p in pen], dtype=np.float32))
+        self.k.zk_penalize(logits.ptr, V, rows_d.ptr, toks_d.ptr, scales_d.ptr, m, self.rt.stream)
