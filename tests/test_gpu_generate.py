@@ -146,7 +146,7 @@ def test_sampled_requests_do_not_depend_on_the_batch(tiny_folders):
         assert tok == P.sample(z[len(prompts[3]) - 1 + i], uniform(7, i), temperature=0.8)
 
 
-def test_top_k_top_p_and_penalty_rows_go_through_the_host_sampler(tiny_folders):
+def test_top_k_top_p_and_penalty_rows(tiny_folders):
     from zse_amd.engine.engine import Engine
     from zse_amd.sampling import SamplingParams
     folder = tiny_folders[("A", "float32")]
@@ -162,7 +162,25 @@ def test_top_k_top_p_and_penalty_rows_go_through_the_host_sampler(tiny_folders):
     assert len(set(pen) | set(prompt)) == len(pen) + len(set(prompt))     # nothing is repeated
     stop = eng.generate([prompt], SamplingParams(max_tokens=6, temperature=0.0, stop_tokens=[greedy[-1]]))[0]
     assert stop == greedy[:greedy.index(greedy[-1]) + 1]
+    # all of them together: the same tokens alone and beside other requests, and each token is what
+    # the host implementation draws from logits of the same position
+    from zse_amd.engine.runner import StepEntry
+    from zse_amd.sampling import sample_host, uniform
+    mixed = SamplingParams(max_tokens=10, temperature=0.8, top_k=7, top_p=0.85, repetition_penalty=1.3, seed=11)
+    alone = eng.generate([prompt], mixed)[0]
+    others = [random_tokens(512, n, 30 + n) for n in (3, 14)]
+    batch = eng.generate([others[0], prompt, others[1]],
+                         [SamplingParams(max_tokens=10, temperature=0.0), mixed,
+                          SamplingParams(max_tokens=10, temperature=1.2, top_p=0.5, seed=2)])
+    assert batch[1] == alone
     eng.close()
+    from gpu_util import make_runner
+    runner = make_runner(folder, "float32", page_size=4, cache_tokens=64, max_seqs=2, max_batch_tokens=64,
+                         max_model_len=64)
+    seq = prompt + alone
+    z = runner.step([StepEntry("s", seq, list(range(len(seq))))])
+    for i, tok in enumerate(alone):
+        assert tok == sample_host(z[len(prompt) - 1 + i], mixed, uniform(11, i), set(seq[:len(prompt) + i]))
 
 
 def test_zse_generate_command(tiny_folders, tmp_path):
