@@ -67,8 +67,8 @@ def test_greedy_generation_bfloat16(tiny_folders):
             toks.append(t)
 
 
-@pytest.mark.parametrize("temperature", [0.0, 0.9])
-def test_runs_of_steps_without_the_host_give_the_same_tokens(tiny_folders, temperature):
+@pytest.mark.parametrize("temperature,top_k,top_p", [(0.0, 0, 1.0), (0.9, 0, 1.0), (0.9, 6, 0.8)])
+def test_runs_of_steps_without_the_host_give_the_same_tokens(tiny_folders, temperature, top_k, top_p):
     """Decoding several steps in a row before the host reads an id (the ids go from step to step
     on the device) gives what step-by-step decoding gives: same tokens, same ends by length and
     by stop token (found late: the output is cut back to it), also when pages run short in the
@@ -84,7 +84,7 @@ def test_runs_of_steps_without_the_host_give_the_same_tokens(tiny_folders, tempe
         eng = Engine(folder, dtype="float32", block_size=8, num_blocks=num_blocks, max_batch_tokens=32,
                      max_batch_seqs=4, prefill_chunk_size=7, max_seq_len=128, decode_run=decode_run)
         reqs = [eng.add_request(p, SamplingParams(max_tokens=m, temperature=temperature, seed=11 + i,
-                                                  stop_tokens=stops))
+                                                  top_k=top_k, top_p=top_p, stop_tokens=stops))
                 for i, (p, m) in enumerate(zip(prompts, (21, 5, 30, 13)))]
         eng.run()
         out = [(list(r.output_tokens), r.finish_reason) for r in reqs]

@@ -55,9 +55,14 @@ class SamplingParams:
 
     @property
     def plain(self) -> bool:
-        """Greedy or temperature alone: nothing but the logits and a uniform number is needed,
-        so runs of steps can be enqueued without the host in between."""
+        """Greedy or temperature alone."""
         return self.repetition_penalty == 1.0 and (self.greedy or (self.top_k == 0 and self.top_p >= 1.0))
+
+    @property
+    def stateless(self) -> bool:
+        """Nothing but the logits and a uniform number is needed (no penalty, which looks at the
+        tokens so far), so runs of steps can be enqueued without the host in between."""
+        return self.repetition_penalty == 1.0
 
 
 def _mix64(z: int) -> int:
@@ -152,9 +157,9 @@ class DeviceSampler:
     RING = 16       # results that may be on their way to the host at a time
 
     def can_defer(self, rows: Sequence[dict]) -> bool:
-        """True when ``sample_deferred`` serves these rows: nothing but greedy or temperature,
-        and all of one kind."""
-        if not rows or len(rows) > self.max_rows or not all(r["params"].plain for r in rows):
+        """True when ``sample_deferred`` serves these rows: no penalties, and all greedy or all
+        drawn."""
+        if not rows or len(rows) > self.max_rows or not all(r["params"].stateless for r in rows):
             return False
         kinds = {bool(r["params"].greedy) for r in rows}
         return len(kinds) == 1
@@ -169,6 +174,10 @@ class DeviceSampler:
         if self._run_greedy:
             return
         self.rt.copy_h2d(self.temp.ptr, np.array([r["params"].temperature for r in rows], dtype=np.float32))
+        self._run_cut = any(r["params"].top_k > 0 or r["params"].top_p < 1.0 for r in rows)
+        if self._run_cut:
+            self.rt.copy_h2d(self.top_k.ptr, np.array([r["params"].top_k for r in rows], dtype=np.int32))
+            self.rt.copy_h2d(self.top_p.ptr, np.array([r["params"].top_p for r in rows], dtype=np.float32))
         flat = np.ascontiguousarray(np.asarray(us, dtype=np.float64).reshape(len(us), n))
         if getattr(self, "_run_u", None) is None or self._run_u.shape[0] < flat.size:
             self._run_u = self.rt.empty((max(flat.size, self.max_rows * 8),), F64)
@@ -184,7 +193,11 @@ class DeviceSampler:
             k.zk_argmax(logits.ptr, self.ids.ptr, n, V, self.scratch.ptr, rt.stream)
             dev = self.ids
         else:
-            k.zk_sample(logits.ptr, self.temp.ptr, self._run_u.ptr + step_in_run * n * 8, None, None,
+            if self._run_cut:
+                k.zk_sample_cutoff(logits.ptr, self.temp.ptr, self.top_k.ptr, self.top_p.ptr, self.keep_from.ptr,
+                                   self.keep_ties.ptr, n, V, rt.stream)
+            k.zk_sample(logits.ptr, self.temp.ptr, self._run_u.ptr + step_in_run * n * 8,
+                        self.keep_from.ptr if self._run_cut else None, self.keep_ties.ptr if self._run_cut else None,
                         self.ids2.ptr, n, V, self.scratch.ptr, rt.stream)
             dev = self.ids2
         if getattr(self, "_ring", None) is None:
@@ -218,8 +231,7 @@ class DeviceSampler:
             u = np.array([r["u"] for r in rows], dtype=np.float64)
             rt.copy_h2d(self.temp.ptr, t)
             rt.copy_h2d(self.u.ptr, u)
-            cut = any(not g and not r["params"].plain and (r["params"].top_k > 0 or r["params"].top_p < 1.0)
-                      for r, g in zip(rows, greedy))
+            cut = any(not g and (r["params"].top_k > 0 or r["params"].top_p < 1.0) for r, g in zip(rows, greedy))
             if cut:
                 rt.copy_h2d(self.top_k.ptr, np.array([0 if g else r["params"].top_k for r, g in zip(rows, greedy)],
                                                      dtype=np.int32))
