@@ -80,9 +80,9 @@ def test_runs_of_steps_without_the_host_give_the_same_tokens(tiny_folders, tempe
     folder = tiny_folders[("B", "float32")]
     prompts = [random_tokens(cfg["vocab_size"], n, 70 + n) for n in (3, 9, 14, 6)]
 
-    def run(decode_run, num_blocks, stops):
+    def run(decode_run, num_blocks, stops, seqs=4):
         eng = Engine(folder, dtype="float32", block_size=8, num_blocks=num_blocks, max_batch_tokens=32,
-                     max_batch_seqs=4, prefill_chunk_size=7, max_seq_len=128, decode_run=decode_run)
+                     max_batch_seqs=seqs, prefill_chunk_size=7, max_seq_len=128, decode_run=decode_run)
         reqs = [eng.add_request(p, SamplingParams(max_tokens=m, temperature=temperature, seed=11 + i,
                                                   top_k=top_k, top_p=top_p, stop_tokens=stops))
                 for i, (p, m) in enumerate(zip(prompts, (21, 5, 30, 13)))]
@@ -108,6 +108,9 @@ def test_runs_of_steps_without_the_host_give_the_same_tokens(tiny_folders, tempe
     tight, st1 = run(1, 8, ())
     assert st1.preemptions > 0 and [o for o, _ in tight] == [o for o, _ in base]
     assert run(4, 8, ())[0] == tight
+    # more requests than places: runs go on while others wait, and the waiting ones get their turn
+    few, st2 = run(4, 64, (stop,), seqs=2)
+    assert few == want and st2.steps < run(1, 64, (stop,), seqs=2)[1].steps + 8
 
 
 def test_sampled_requests_do_not_depend_on_the_batch(tiny_folders):

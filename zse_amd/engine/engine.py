@@ -122,9 +122,11 @@ class Engine:
 
     def _run_length(self, plan: StepPlan) -> int:
         """How many steps can follow each other before the host reads an id: every request
-        decodes, is sampled on the device in one manner, nobody waits to be admitted, and
-        nobody reaches its length before the run's last step."""
-        if self.decode_run < 2 or self.scheduler.waiting or plan.preempted or plan.failed:
+        decodes (so whoever waits could not be admitted to this step), is sampled on the
+        device in one manner, and nobody reaches its length before the run's last step.  The
+        run ends early when a later step's plan differs, a newcomer included; a request that
+        waits only for a stop token found late waits a few steps longer."""
+        if self.decode_run < 2 or plan.preempted or plan.failed:
             return 1
         if not all(s.count == 1 and s.sample and s.request.state == RequestState.DECODING for s in plan.items):
             return 1
