@@ -207,11 +207,18 @@ __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
         load4<act_t>(s + i, v[j]);
       } else {
         load4<float>(sf + i, v[j]);
-        for (int p = 1; p < parts; p++) {
-          float t[4];
-          load4<float>(sf + p * plane + i, t);
+        // four planes a turn, their loads issued together; a plane past the last is read from
+        // the last and not added
+        for (int p0 = 1; p0 < parts; p0 += 4) {
+          float t[4][4];
 #pragma unroll
-          for (int e = 0; e < 4; e++) v[j][e] += t[e];
+          for (int q = 0; q < 4; q++) load4<float>(sf + (size_t)min(p0 + q, parts - 1) * plane + i, t[q]);
+#pragma unroll
+          for (int q = 0; q < 4; q++)
+            if (p0 + q < parts) {
+#pragma unroll
+              for (int e = 0; e < 4; e++) v[j][e] += t[q][e];
+            }
         }
 #pragma unroll
         for (int e = 0; e < 4; e++) v[j][e] = to_f32(from_f32<act_t>(v[j][e]));
