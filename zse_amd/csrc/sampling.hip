@@ -256,12 +256,13 @@ __global__ __launch_bounds__(256) void sample_pick_kernel(
 // k-th largest logit on (all its ties, orchestrator/sampler.py:146-156), top-p then the fewest
 // of the largest that hold a share p of what is left, equal ones in the order of their indices
 // (:186-203).  The value is found by narrowing a range of keys (the logits' bits, made to sort
-// like the numbers) by eight bits a pass: a histogram over the range, by count for top-k, by
-// weight exp((z - max) / T) for top-p, walked from the top.  Every wave has a histogram of its
-// own in LDS, so that lanes of different waves never meet at one counter.  Weights are added up
-// as 64-bit integers (units of 2^-44 of the largest logit's weight): integer additions in LDS
-// are one instruction where additions of doubles are a loop, and their sum does not depend on
-// the order, so the cut-off is the same on every run.
+// like the numbers) by eight bits a pass, four passes for each of the two: a histogram over the
+// range, by count for top-k, by weight exp((z - max) / T) for top-p, walked from the top.  A
+// pass is two launches: 16 blocks a row fill histograms of their slices (each wave one of its
+// own in LDS, so that lanes of different waves never meet at one counter), one block a row adds
+// them up and walks.  Weights are added up as 64-bit integers (units of 2^-44 of the largest
+// logit's weight): integer additions are one instruction where additions of doubles are a loop,
+// and their sum does not depend on the order, so the cut-off is the same on every run.
 __device__ __forceinline__ unsigned int key_of(float v) {
   const unsigned int b = __float_as_uint(v);
   return v != v ? 0u : ((b & 0x80000000u) ? ~b : (b | 0x80000000u));
@@ -274,178 +275,152 @@ __device__ __forceinline__ unsigned long long weight_of(float x) {
   return (unsigned long long)((double)__expf(x) * 17592186044416.0);
 }
 
-#define SC_WAVES 16
-// Every logit of a row through f, four to a load where the row allows it (the block has one CU's
-// share of the memory system to itself, so it wants many loads in flight).
-template <typename F>
-__device__ __forceinline__ void each_logit(const float* __restrict__ z, int V, int tid, F f) {
-  if (V % 4 == 0 && (uintptr_t)z % 16 == 0) {
-    const float4* z4 = (const float4*)z;
-    int i = tid;
-    for (; i + 64 * SC_WAVES < V / 4; i += 2 * 64 * SC_WAVES) {
-      const float4 a = z4[i], b = z4[i + 64 * SC_WAVES];
-      f(a.x); f(a.y); f(a.z); f(a.w);
-      f(b.x); f(b.y); f(b.z); f(b.w);
-    }
-    if (i < V / 4) {
-      const float4 a = z4[i];
-      f(a.x); f(a.y); f(a.z); f(a.w);
-    }
+#define SC_SLICES 16
+struct CutState {
+  unsigned int lo, hi;            // the range of keys still in question (inclusive)
+  unsigned int floor_key;         // top-p: what top-k left
+  unsigned int count;             // logits with the key the range has narrowed to
+  unsigned long long above;       // count or weight of the keys above the range
+  unsigned long long target;
+  float mx, inv_t, share;
+  int by_weight, active, passes;
+};
+struct CutHist {
+  unsigned int cnt[256];
+  unsigned long long w[256];
+};
+__device__ __forceinline__ int cut_shift(unsigned int lo, unsigned int hi) {
+  const unsigned int width = hi - lo;
+  return width < 256u ? 0 : 32 - __builtin_clz(width) - 8;
+}
+
+// Starts a row's search: stage 0 = top-k over all keys, stage 1 = top-p over what top-k left.
+__global__ void cutoff_begin_kernel(CutState* __restrict__ st, const float* __restrict__ pv,
+                                    const float* __restrict__ temperature, const int* __restrict__ top_k,
+                                    const float* __restrict__ top_p, int V, int stage, int rows) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  CutState& c = st[r];
+  if (stage == 0) {
+    const int k = top_k ? top_k[r] : 0;
+    c.mx = row_max(pv, r);
+    c.inv_t = 1.f / temperature[r];
+    c.floor_key = 0u;
+    c.lo = 0u;
+    c.hi = 0xffffffffu;
+    c.above = 0;
+    c.count = 0;
+    c.target = (unsigned long long)max(k, 0);
+    c.by_weight = 0;
+    c.passes = 0;
+    c.active = k > 0 && k < V;
   } else {
-    for (int i = tid; i < V; i += 64 * SC_WAVES) f(z[i]);
+    const float p = top_p ? top_p[r] : 1.f;
+    if (c.active) c.floor_key = c.lo;      // top-k ran: its key is the floor
+    c.lo = c.floor_key;
+    c.hi = 0xffffffffu;
+    c.above = 0;
+    c.count = 0;
+    c.share = p;
+    c.by_weight = 1;
+    c.passes = 0;
+    c.active = p < 1.f;
   }
 }
 
-__global__ __launch_bounds__(64 * SC_WAVES) void sample_cutoff_kernel(
-    const float* __restrict__ logits, int V, const float* __restrict__ temperature, const int* __restrict__ top_k,
-    const float* __restrict__ top_p, float* __restrict__ keep_from, int* __restrict__ keep_ties) {
-  __shared__ unsigned int h_cnt[SC_WAVES][256];
-  __shared__ unsigned long long h_w[SC_WAVES][256];
-  __shared__ unsigned int s_lo, s_hi, s_kmin, s_kmax, s_count;
-  __shared__ unsigned long long s_above, s_target;
-  __shared__ float s_red[SC_WAVES];
-  const int r = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const float* z = logits + (size_t)r * V;
-  const int k = top_k ? top_k[r] : 0;
-  const float p = top_p ? top_p[r] : 1.f;
-  const bool use_k = k > 0 && k < V, use_p = p < 1.f;
-  if (!use_k && !use_p) {
-    if (tid == 0) {
-      keep_from[r] = -INFINITY;
-      keep_ties[r] = -1;
-    }
-    return;
+__global__ __launch_bounds__(256) void cutoff_hist_kernel(const float* __restrict__ logits, int V,
+                                                          const CutState* __restrict__ st, CutHist* __restrict__ hist) {
+  __shared__ unsigned int h_cnt[4][256];
+  __shared__ unsigned long long h_w[4][256];
+  const int row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x, wave = tid >> 6;
+  const CutState c = st[row];
+  if (!c.active || (c.lo == c.hi && c.passes > 0)) return;
+  for (int i = tid; i < 4 * 256; i += 256) {
+    (&h_cnt[0][0])[i] = 0;
+    (&h_w[0][0])[i] = 0;
   }
-  const float inv_t = 1.f / temperature[r];
-  // the row's largest logit and the range of its keys
-  float mx = -INFINITY;
-  unsigned int kmin = 0xffffffffu, kmax = 0u;
-  each_logit(z, V, tid, [&](float v) {
+  __syncthreads();
+  const float* z = logits + (size_t)row * V;
+  const int per = (V + SC_SLICES - 1) / SC_SLICES;
+  const int b = slice * per, e = min(V, b + per);
+  const int shift = cut_shift(c.lo, c.hi);
+  for (int i = b + tid; i < e; i += 256) {
+    const float v = z[i];
     const unsigned int key = key_of(v);
-    mx = fmaxf(mx, v);
-    kmin = min(kmin, key);
-    kmax = max(kmax, key);
-  });
-  mx = wave_max(mx);
-  for (int o = 32; o > 0; o >>= 1) {
-    kmin = min(kmin, (unsigned int)__shfl_xor((int)kmin, o, 64));
-    kmax = max(kmax, (unsigned int)__shfl_xor((int)kmax, o, 64));
-  }
-  if (tid == 0) {
-    s_kmin = 0xffffffffu;
-    s_kmax = 0u;
+    if (key < c.lo || key > c.hi) continue;
+    const unsigned int bucket = (key - c.lo) >> shift;
+    atomicAdd(&h_cnt[wave][bucket], 1u);
+    if (c.by_weight) atomicAdd(&h_w[wave][bucket], weight_of((v - c.mx) * c.inv_t));
   }
   __syncthreads();
-  if (lane == 0) {
-    s_red[wave] = mx;
-    atomicMin(&s_kmin, kmin);
-    atomicMax(&s_kmax, kmax);
-  }
-  __syncthreads();
-  mx = s_red[0];
-  for (int w = 1; w < SC_WAVES; w++) mx = fmaxf(mx, s_red[w]);
-  kmin = s_kmin;
-  kmax = s_kmax;
-  __syncthreads();
+  CutHist& out = hist[(size_t)row * SC_SLICES + slice];
+  out.cnt[tid] = h_cnt[0][tid] + h_cnt[1][tid] + h_cnt[2][tid] + h_cnt[3][tid];
+  out.w[tid] = h_w[0][tid] + h_w[1][tid] + h_w[2][tid] + h_w[3][tid];
+}
 
-  // Narrows [s_lo, s_hi] to one key: the key at which, walking down from the largest, the
-  // count (by_weight false) of the keys >= floor reaches `target`, or their weight the share
-  // `share` of its total (which the first pass, over all of them, gives: s_target).  Leaves in
-  // s_above what lies above that key and in s_count how many logits have it.
-  auto narrow = [&](bool by_weight, unsigned int floor_key, unsigned long long target, float share) {
-    if (tid == 0) {
-      s_lo = max(kmin, floor_key);
-      s_hi = kmax;
-      s_above = 0;
-      s_count = 0;
-      s_target = target;
+// Adds the slices' histograms up and walks them from the top: to the bucket at which the count
+// (or the weight) of the keys from the floor on reaches the target; the range becomes that bucket.
+__global__ __launch_bounds__(256) void cutoff_walk_kernel(CutState* __restrict__ st, const CutHist* __restrict__ hist) {
+  __shared__ unsigned int cnt[256];
+  __shared__ unsigned long long w[256];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  CutState& c = st[row];
+  if (!c.active || (c.lo == c.hi && c.passes > 0)) return;
+  unsigned int n = 0;
+  unsigned long long sw = 0;
+  for (int q = 0; q < SC_SLICES; q++) {
+    n += hist[(size_t)row * SC_SLICES + q].cnt[tid];
+    sw += hist[(size_t)row * SC_SLICES + q].w[tid];
+  }
+  cnt[tid] = n;
+  w[tid] = sw;
+  __syncthreads();
+  if (tid != 0) return;
+  if (c.by_weight && c.passes == 0) {          // the first pass covers everything top-k left: its sum is the whole
+    unsigned long long total = 0;
+    for (int b = 0; b < 256; b++) total += w[b];
+    c.target = (unsigned long long)ceil((double)c.share * (double)total);
+  }
+  const int shift = cut_shift(c.lo, c.hi);
+  unsigned long long acc = c.above;
+  int pick = -1, lowest = -1;
+  for (int b = 255; b >= 0; b--) {
+    if (cnt[b] == 0) continue;
+    lowest = b;
+    const unsigned long long here = c.by_weight ? w[b] : (unsigned long long)cnt[b];
+    if (acc + here >= c.target) {
+      pick = b;
+      break;
     }
-    __syncthreads();
-    bool counted = false;
-    while (true) {
-      const unsigned int lo = s_lo, hi = s_hi;
-      if (lo == hi && counted) break;
-      const unsigned int width = hi - lo;                       // inclusive range minus one
-      const int shift = width < 256u ? 0 : 32 - __builtin_clz(width) - 8;
-      for (int i = lane; i < 256; i += 64) {
-        h_cnt[wave][i] = 0;
-        h_w[wave][i] = 0;
-      }
-      __syncthreads();
-      each_logit(z, V, tid, [&](float v) {
-        const unsigned int key = key_of(v);
-        if (key < lo || key > hi) return;
-        const unsigned int b = (key - lo) >> shift;
-        atomicAdd(&h_cnt[wave][b], 1u);
-        if (by_weight) atomicAdd(&h_w[wave][b], weight_of((v - mx) * inv_t));
-      });
-      __syncthreads();
-      for (int i = tid; i < 256; i += 64 * SC_WAVES) {
-        unsigned int c = 0;
-        unsigned long long w = 0;
-        for (int q = 0; q < SC_WAVES; q++) {
-          c += h_cnt[q][i];
-          w += h_w[q][i];
-        }
-        h_cnt[0][i] = c;
-        h_w[0][i] = w;
-      }
-      __syncthreads();
-      if (tid == 0) {
-        if (by_weight && !counted) {
-          unsigned long long total = 0;
-          for (int b = 0; b < 256; b++) total += h_w[0][b];
-          s_target = (unsigned long long)ceil((double)share * (double)total);
-        }
-        const unsigned long long target = s_target;
-        unsigned long long acc = s_above;
-        int pick = -1, lowest = -1;
-        for (int b = 255; b >= 0; b--) {
-          if (h_cnt[0][b] == 0) continue;
-          lowest = b;
-          const unsigned long long here = by_weight ? h_w[0][b] : (unsigned long long)h_cnt[0][b];
-          if (acc + here >= target) {
-            pick = b;
-            break;
-          }
-          acc += here;
-        }
-        if (pick < 0) {           // rounding: the whole range falls short of the target; its lowest keys then
-          pick = lowest;
-          acc -= by_weight ? h_w[0][pick] : (unsigned long long)h_cnt[0][pick];
-        }
-        s_above = acc;
-        s_count = h_cnt[0][pick];
-        const unsigned long long first = (unsigned long long)lo + ((unsigned long long)pick << shift);
-        s_lo = (unsigned int)first;
-        s_hi = (unsigned int)min((unsigned long long)hi, first + ((1ull << shift) - 1ull));
-      }
-      __syncthreads();
-      counted = true;
-    }
-  };
+    acc += here;
+  }
+  if (pick < 0) {             // rounding: the whole range falls short of the target; its lowest keys then
+    pick = max(lowest, 0);
+    acc -= c.by_weight ? w[pick] : (unsigned long long)cnt[pick];
+  }
+  const unsigned long long first = (unsigned long long)c.lo + ((unsigned long long)pick << shift);
+  c.above = acc;
+  c.count = cnt[pick];
+  c.hi = (unsigned int)min((unsigned long long)c.hi, first + ((1ull << shift) - 1ull));
+  c.lo = (unsigned int)first;
+  c.passes++;
+}
 
-  unsigned int floor_key = 0u;
-  int ties = -1;
-  if (use_k) {
-    narrow(false, 0u, (unsigned long long)k, 0.f);
-    floor_key = s_lo;
-    __syncthreads();
-  }
-  if (use_p) {
-    narrow(true, floor_key, 0, p);
-    if (tid == 0) {
-      const unsigned long long each = weight_of((value_of(s_lo) - mx) * inv_t);
-      const unsigned long long missing = s_target > s_above ? s_target - s_above : 0;
-      unsigned long long c = each > 0 ? (missing + each - 1) / each : 1;
-      c = max(1ull, min(c, (unsigned long long)s_count));
-      ties = (int)c;
-    }
-    floor_key = s_lo;
-  }
-  if (tid == 0) {
-    keep_from[r] = value_of(floor_key);
-    keep_ties[r] = ties;
+__global__ void cutoff_end_kernel(const CutState* __restrict__ st, float* __restrict__ keep_from,
+                                  int* __restrict__ keep_ties, int rows) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  const CutState& c = st[r];
+  if (c.active) {             // top-p ran: the first few of the ties at its key
+    const unsigned long long each = weight_of((value_of(c.lo) - c.mx) * c.inv_t);
+    const unsigned long long missing = c.target > c.above ? c.target - c.above : 0;
+    unsigned long long n = each > 0 ? (missing + each - 1) / each : 1;
+    n = max(1ull, min(n, (unsigned long long)c.count));
+    keep_from[r] = value_of(c.lo);
+    keep_ties[r] = (int)n;
+  } else {                    // top-k alone (all ties of its key) or nothing
+    keep_from[r] = c.floor_key ? value_of(c.floor_key) : -INFINITY;
+    keep_ties[r] = -1;
   }
 }
 
@@ -505,13 +480,36 @@ int zk_sample(const float* logits, const float* temperature, const double* unifo
 }
 
 // top_k[r] <= 0 or >= V: no top-k; top_p[r] >= 1: no top-p.  Either pointer may be null.
+// scratch: zk_sample_cutoff_scratch_bytes(rows).
+size_t zk_sample_cutoff_scratch_bytes(int rows) {
+  return (size_t)rows * (sizeof(CutState) + SC_SLICES * sizeof(CutHist) + AM_SLICES * 8) + 64;
+}
+
 int zk_sample_cutoff(const float* logits, const float* temperature, const int* top_k, const float* top_p,
-                     float* keep_from, int* keep_ties, int rows, int V, void* stream) {
+                     float* keep_from, int* keep_ties, int rows, int V, void* scratch, void* stream) {
   ZK_REQUIRE(rows >= 0 && V > 0, "zk_sample_cutoff: bad sizes");
+  ZK_REQUIRE(rows <= 65535, "zk_sample_cutoff: too many rows");
   ZK_REQUIRE(temperature && keep_from && keep_ties, "zk_sample_cutoff: temperature and outputs are needed");
+  ZK_REQUIRE(scratch != nullptr && (uintptr_t)scratch % 8 == 0, "zk_sample_cutoff: no scratch buffer");
   if (rows == 0) return 0;
-  sample_cutoff_kernel<<<rows, 64 * SC_WAVES, 0, (hipStream_t)stream>>>(logits, V, temperature, top_k, top_p,
-                                                                        keep_from, keep_ties);
+  hipStream_t s = (hipStream_t)stream;
+  CutHist* hist = (CutHist*)scratch;
+  CutState* st = (CutState*)(hist + (size_t)rows * SC_SLICES);
+  float* pv = (float*)(st + rows);
+  int* pi = (int*)(pv + (size_t)rows * AM_SLICES);
+  argmax_slices_kernel<<<dim3(AM_SLICES, rows), 256, 0, s>>>(logits, V, pv, pi);
+  for (int stage = 0; stage < 2; stage++) {
+    if (stage == 0 && top_k == nullptr) {
+      // no top-k anywhere: the state still has to be set up
+    }
+    cutoff_begin_kernel<<<(rows + 63) / 64, 64, 0, s>>>(st, pv, temperature, top_k, top_p, V, stage, rows);
+    if ((stage == 0 && top_k == nullptr) || (stage == 1 && top_p == nullptr)) continue;
+    for (int pass = 0; pass < 4; pass++) {          // 32 bits of key, eight a pass
+      cutoff_hist_kernel<<<dim3(SC_SLICES, rows), 256, 0, s>>>(logits, V, st, hist);
+      cutoff_walk_kernel<<<rows, 256, 0, s>>>(st, hist);
+    }
+  }
+  cutoff_end_kernel<<<(rows + 63) / 64, 64, 0, s>>>(st, keep_from, keep_ties, rows);
   return zk_launch_status("zk_sample_cutoff");
 }
 

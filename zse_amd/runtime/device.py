@@ -155,7 +155,7 @@ KERNEL_SIGNATURES = {
                            _I, _I, _VP],
     "zk_argmax": [_VP, _VP, _I, _I, _VP, _VP],
     "zk_sample": [_VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP],
-    "zk_sample_cutoff": [_VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP],
+    "zk_sample_cutoff": [_VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP],
     "zk_penalize": [_VP, _I, _VP, _VP, _VP, _I, _VP],
 }
 # present only in the bf16 library
@@ -187,6 +187,10 @@ class KernelLibrary:
             fn.argtypes = args
             fn.restype = C.c_int
             setattr(self, name, self._wrap(name, fn))
+        for name in ("zk_sample_scratch_bytes", "zk_sample_cutoff_scratch_bytes"):
+            fn = getattr(self._dll, name)
+            fn.restype, fn.argtypes = C.c_size_t, [_I]
+            setattr(self, name, fn)
         if dtype == BF16:
             self._dll.zk_attention_bf16_supports.restype = C.c_int
             self._dll.zk_attention_bf16_supports.argtypes = [_I, _I, _I, _I]

@@ -146,7 +146,8 @@ class DeviceSampler:
         self.ids2 = rt.empty((max_rows,), I32)
         self.temp = rt.empty((max_rows,), F32)
         self.u = rt.empty((max_rows,), F64)
-        self.scratch = rt.empty((max_rows * 64 * 5,), F32)  # per row 64 slices: a double, a float, an int
+        self.scratch = rt.empty(((kernels.zk_sample_scratch_bytes(max_rows) + 3) // 4,), F32)
+        self.cut_scratch = None                             # histograms of the cut-off search, on first use
         self.top_k = rt.empty((max_rows,), I32)
         self.top_p = rt.empty((max_rows,), F32)
         self.keep_from = rt.empty((max_rows,), F32)
@@ -194,8 +195,7 @@ class DeviceSampler:
             dev = self.ids
         else:
             if self._run_cut:
-                k.zk_sample_cutoff(logits.ptr, self.temp.ptr, self.top_k.ptr, self.top_p.ptr, self.keep_from.ptr,
-                                   self.keep_ties.ptr, n, V, rt.stream)
+                self._cutoff(logits, n, V)
             k.zk_sample(logits.ptr, self.temp.ptr, self._run_u.ptr + step_in_run * n * 8,
                         self.keep_from.ptr if self._run_cut else None, self.keep_ties.ptr if self._run_cut else None,
                         self.ids2.ptr, n, V, self.scratch.ptr, rt.stream)
@@ -237,13 +237,20 @@ class DeviceSampler:
                                                      dtype=np.int32))
                 rt.copy_h2d(self.top_p.ptr, np.array([1.0 if g else r["params"].top_p for r, g in zip(rows, greedy)],
                                                      dtype=np.float32))
-                k.zk_sample_cutoff(logits.ptr, self.temp.ptr, self.top_k.ptr, self.top_p.ptr, self.keep_from.ptr,
-                                   self.keep_ties.ptr, n, V, rt.stream)
+                self._cutoff(logits, n, V)
             k.zk_sample(logits.ptr, self.temp.ptr, self.u.ptr, self.keep_from.ptr if cut else None,
                         self.keep_ties.ptr if cut else None, self.ids2.ptr, n, V, self.scratch.ptr, rt.stream)
         g = rt.download(self.ids.rows(0, n)) if any(greedy) else None
         s = rt.download(self.ids2.rows(0, n)) if not all(greedy) else None
         return [int(g[i]) if greedy[i] else int(s[i]) for i in range(n)]
+
+    def _cutoff(self, logits, n: int, V: int) -> None:
+        """top-k / top-p of the rows (``self.top_k``, ``self.top_p``) as ``keep_from`` / ``keep_ties``."""
+        from ..runtime.device import F32
+        if self.cut_scratch is None:
+            self.cut_scratch = self.rt.empty(((self.k.zk_sample_cutoff_scratch_bytes(self.max_rows) + 3) // 4,), F32)
+        self.k.zk_sample_cutoff(logits.ptr, self.temp.ptr, self.top_k.ptr, self.top_p.ptr, self.keep_from.ptr,
+                                self.keep_ties.ptr, n, V, self.cut_scratch.ptr, self.rt.stream)
 
     def _penalize(self, logits, V: int, pen) -> None:
         from ..runtime.device import F32, I32
