@@ -663,3 +663,27 @@ def test_top_k_top_p_and_penalty_on_the_device(rt, V, ties):
         got = sampler.sample(rt.upload(z), rows)                 # the penalty changes the logits in place: a fresh copy
         want = [sample_host(z[i], r["params"], r["u"], r["past"]) for i, r in enumerate(rows)]
         assert got == want, [(i, combos[i], g, w) for i, (g, w) in enumerate(zip(got, want)) if g != w]
+
+
+def test_cut_offs_on_awkward_rows(rt):
+    """All logits equal, two values only, minus infinity among them, a spread that leaves most
+    weights at zero, a share that only the largest logit holds: the device still draws what
+    the host implementation draws."""
+    from zse_amd.sampling import DeviceSampler, SamplingParams, sample_host, uniform
+    rng = np.random.default_rng(9)
+    V = 1000
+    flat = np.zeros(V, np.float32)
+    two = np.where(rng.random(V) < 0.3, 2.0, -1.0).astype(np.float32)
+    holes = (rng.normal(size=V) * 2).astype(np.float32)
+    holes[rng.random(V) < 0.5] = -np.inf
+    wide = (rng.normal(size=V) * 3000).astype(np.float32)
+    rows_z = [flat, two, holes, wide]
+    combos = [dict(top_k=10), dict(top_p=0.4995), dict(top_k=300, top_p=0.9), dict(top_p=1e-6), dict(top_k=999, top_p=0.9995)]      # (no share that a whole number of equal logits holds exactly)
+    z = np.stack([r for r in rows_z for _ in combos])
+    params = [SamplingParams(temperature=0.9, **c) for _ in rows_z for c in combos]
+    sampler = DeviceSampler(rt, rt.kernels("float32"), len(params))
+    for trial in range(4):
+        rows = [{"params": p_, "u": uniform(trial, i), "past": ()} for i, p_ in enumerate(params)]
+        got = sampler.sample(rt.upload(z), rows)
+        want = [sample_host(z[i], r["params"], r["u"]) for i, r in enumerate(rows)]
+        assert got == want, [(i, g, w) for i, (g, w) in enumerate(zip(got, want)) if g != w]
