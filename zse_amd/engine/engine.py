@@ -68,7 +68,7 @@ class Engine:
         # Steps of single tokens in a row that are enqueued before the host looks at the ids
         # they produced (1: look after every step).  The ids are fed from step to step on the
         # device; a stop token found afterwards cuts the request's output back to it.
-        self.decode_run = max(1, int(decode_run))
+        self.decode_run = max(1, min(int(decode_run), DeviceSampler.RING))     # results on their way at a time
         self._next_plan: Optional[StepPlan] = None
 
     # ---- requests
