@@ -921,6 +921,9 @@ extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int 
   (gated ? (exact ? ZK_TILE_(W_, M_, N_, true, true) : ZK_TILE_(W_, M_, N_, true, false))             \
          : (exact ? ZK_TILE_(W_, M_, N_, false, true) : ZK_TILE_(W_, M_, N_, false, false)))
   if (wide) return ZK_TILE(2, 2, 4);
+  // few rows: 128 x 128 tiles leave half of the CUs or more without a block; 64-row tiles
+  // make twice as many
+  if (nb_small <= 128 && ksplit == 1 && M > 64) return ZK_TILE(1, 2, 2);
   return ZK_TILE(2, 2, 2);
 #undef ZK_TILE
 #undef ZK_TILE_
