@@ -908,22 +908,24 @@ extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int 
   const bool exact = K % GT_BK == 0;
   // Few small blocks: split K over blocks until about 320 blocks exist, a range no shorter than
   // 8 k tiles, and the partial sums (4 M N bytes a range, written and read) no more than W.
-  int ksplit = 1;
-  if (!wide && nb_small < 160) {
-    ksplit = (int)(320 / nb_small);
-    ksplit = min(ksplit, (K + GT_BK - 1) / GT_BK / 8);
-    ksplit = min(ksplit, K / (4 * M));
-    ksplit = max(ksplit, 1);
-  }
+  auto ranges = [&](long blocks) {
+    int ks = (int)(320 / blocks);
+    ks = min(ks, (K + GT_BK - 1) / GT_BK / 8);
+    ks = min(ks, K / (4 * M));
+    return max(ks, 1);
+  };
+  int ksplit = (!wide && nb_small < 160) ? ranges(nb_small) : 1;
+  // few rows and a K too short to split: 128 x 128 tiles leave half of the CUs or more without
+  // a block; 64-row tiles make twice as many (they lose to a split of K where K allows one)
+  const bool low = !wide && M > 64 && nb_small * ksplit <= 128;
+  if (low) ksplit = ranges((long)((M + 63) / 64) * (nb_small / tiles_m));
 #define ZK_TILE_(W_, M_, N_, G_, E_) \
   launch_tile<W_, M_, N_, G_, E_>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, ws, ws_bytes, ksplit, s)
 #define ZK_TILE(W_, M_, N_)                                                                            \
   (gated ? (exact ? ZK_TILE_(W_, M_, N_, true, true) : ZK_TILE_(W_, M_, N_, true, false))             \
          : (exact ? ZK_TILE_(W_, M_, N_, false, true) : ZK_TILE_(W_, M_, N_, false, false)))
   if (wide) return ZK_TILE(2, 2, 4);
-  // few rows: 128 x 128 tiles leave half of the CUs or more without a block; 64-row tiles
-  // make twice as many
-  if (nb_small <= 128 && ksplit == 1 && M > 64) return ZK_TILE(1, 2, 2);
+  if (low) return ZK_TILE(1, 2, 2);
   return ZK_TILE(2, 2, 2);
 #undef ZK_TILE
 #undef ZK_TILE_
