@@ -583,7 +583,7 @@ static bool joinable_by_reader(int N, int ldc, int c_is_f32, int epi) {
 // with a ticket per column block, the last block adding up, was measured three times slower:
 // the device-wide fences it needs write back and invalidate the L2 of every XCD.)
 #define GM_STEPS 8
-#define GM_LD (GM_STEPS * 32 + 8)
+#define GM_LD (GM_STEPS * 32 + 16)
 
 // A lane's results of one strip: rows n = 16 * strip + 4 * kq + i of W, column m = 16 * mt + r of A.
 template <int MT, bool GATED>
