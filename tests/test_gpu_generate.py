@@ -186,6 +186,61 @@ def test_top_k_top_p_and_penalty_rows(tiny_folders):
         assert tok == sample_host(z[len(prompt) - 1 + i], mixed, uniform(11, i), set(seq[:len(prompt) + i]))
 
 
+@pytest.mark.parametrize("seed", [0, 1])
+def test_a_crowd_of_mixed_requests_each_gets_what_it_gets_alone(tiny_folders, seed):
+    """Two dozen requests of random lengths and every manner of sampling, five places, so few
+    pages that some are recomputed, runs of decode steps on: every request ends with the tokens
+    and the reason it ends with when it has the engine to itself."""
+    import random
+    from zse_amd.engine.engine import Engine
+    from zse_amd.sampling import SamplingParams
+    cfg = TINY["B"][0]
+    folder = tiny_folders[("B", "float32")]
+    rnd = random.Random(seed)
+    V = cfg["vocab_size"]
+    prompts, params = [], []
+    for i in range(24):
+        prompts.append(random_tokens(V, rnd.randint(1, 45), 500 + 31 * seed + i))
+        kind = rnd.choice(["greedy", "temp", "topk", "topp", "both", "penalty"])
+        kw = dict(max_tokens=rnd.randint(1, 20), seed=100 + i)
+        if kind == "greedy":
+            kw.update(temperature=0.0)
+        elif kind == "temp":
+            kw.update(temperature=0.9)
+        elif kind == "topk":
+            kw.update(temperature=1.1, top_k=rnd.choice([1, 3, 40]))
+        elif kind == "topp":
+            kw.update(temperature=0.7, top_p=rnd.choice([0.3, 0.9]))
+        elif kind == "both":
+            kw.update(temperature=1.0, top_k=20, top_p=0.8)
+        else:
+            kw.update(temperature=rnd.choice([0.0, 0.8]), repetition_penalty=1.4)
+        if rnd.random() < 0.4:
+            kw.update(stop_tokens=[rnd.randrange(V) for _ in range(40)])
+        params.append(SamplingParams(**kw))
+
+    def run(which, seqs, blocks):
+        eng = Engine(folder, dtype="float32", block_size=8, num_blocks=blocks, max_batch_tokens=48,
+                     max_batch_seqs=seqs, prefill_chunk_size=11, max_seq_len=128, decode_run=4)
+        reqs = [eng.add_request(prompts[i], params[i]) for i in which]
+        eng.run()
+        out = [(list(r.output_tokens), r.finish_reason) for r in reqs]
+        st = eng.stats()
+        assert all(pool.free_pages == pool.num_pages for pool in eng.runner.manager.pools)
+        eng.close()
+        return out, st
+
+    crowd, st = run(range(24), 5, 22)
+    assert st.preemptions > 0, "the pool was meant to be too small for five long requests"
+    roomy = Engine(folder, dtype="float32", block_size=8, num_blocks=64, max_batch_tokens=48, max_batch_seqs=1,
+                   prefill_chunk_size=16, max_seq_len=128, decode_run=1)
+    for i in range(24):
+        r = roomy.add_request(prompts[i], params[i])
+        roomy.run()
+        assert (list(r.output_tokens), r.finish_reason) == crowd[i], (i, params[i])
+    roomy.close()
+
+
 def test_zse_generate_command(tiny_folders, tmp_path):
     from zse_amd.engine.engine import Engine
     cfg = TINY["A"][0]
