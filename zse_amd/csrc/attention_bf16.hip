@@ -535,6 +535,17 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int c0 = lo / span, c1 = pos / span;
   const size_t base = ((size_t)rr * nh + head) * nchunks;
+  const int np = c1 - c0 + 1;
+  // the first partial results of the thread's channel are asked for now: they come in while
+  // the weights are worked out (a part past the last is read from the last and not used)
+  constexpr int PF = 16;
+  const int d0 = min((int)threadIdx.x, hd - 1);
+  float pf[PF];
+  {
+    const float* po = part_o + (base + c0) * hd + d0;
+#pragma unroll
+    for (int c = 0; c < PF; c++) pf[c] = po[(size_t)min(c, np - 1) * hd];
+  }
   float m = -INFINITY;
   for (int c = c0 + threadIdx.x; c <= c1; c += 256) m = fmaxf(m, part_ml[(base + c) * 2]);
   m = wave_max(m);
@@ -551,11 +562,16 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const float* __restri
   l = block_sum(l, red);
   const float inv = 1.f / l;
   __bf16* orow = out + ((size_t)q_start[r] * nh + head) * hd;
-  const int np = c1 - c0 + 1;
   for (int d = threadIdx.x; d < hd; d += 256) {
     const float* po = part_o + (base + c0) * hd + d;
     float acc = 0.f;
     int c = 0;
+    if (d == d0) {                      // the channel whose first parts are here already
+#pragma unroll
+      for (int q = 0; q < PF; q++)
+        if (q < np) acc += pf[q] * wgt[q];
+      c = min(np, PF);
+    }
     for (; c + 4 <= np; c += 4) {       // four loads in flight, summed in part order
       const float v0 = po[(size_t)c * hd], v1 = po[(size_t)(c + 1) * hd];
       const float v2 = po[(size_t)(c + 2) * hd], v3 = po[(size_t)(c + 3) * hd];
