@@ -59,3 +59,13 @@ def test_params_validate():
     assert SamplingParams(temperature=0).greedy and SamplingParams(temperature=1e-7).greedy
     assert SamplingParams(temperature=0.8).plain and not SamplingParams(top_k=5).plain
     assert SamplingParams(temperature=0, top_k=5).plain and not SamplingParams(temperature=0, repetition_penalty=1.2).plain
+
+
+def test_penalty_scales_follow_how_often_a_token_appeared():
+    # once: the penalty itself; n times: penalty ** (1 + log2 n) (reference orchestrator/sampler.py:64-74)
+    from zse_amd.sampling.sampler import apply_repetition_penalty, penalty_scales
+    sc = penalty_scales({3: 1, 5: 2, 9: 8}, 1.5)
+    assert sc[3] == 1.5 and abs(sc[5] - 1.5 ** 2) < 1e-12 and abs(sc[9] - 1.5 ** 4) < 1e-12
+    assert penalty_scales([4, 4, 7], 2.0) == {4: 2.0, 7: 2.0}          # a plain list counts every token once
+    z = apply_repetition_penalty(np.array([2.0, -2.0, 1.0]), {0: 1, 1: 1, 7: 3}, 2.0)
+    assert list(z) == [1.0, -4.0, 1.0]                                  # positive divided, negative multiplied, out of range ignored
