@@ -85,9 +85,11 @@ def lib_path(name: str) -> str:
 def source_digest(name: str) -> str:
     spec = LIBRARIES[name]
     h = hashlib.sha256()
-    for f in sorted(spec["sources"] + ["common.h"]):
+    headers = [f for f in os.listdir(CSRC) if f.endswith(".h")] if os.path.isdir(CSRC) else []
+    for f in sorted(spec["sources"] + headers):
         p = os.path.join(CSRC, f)
         if os.path.isfile(p):
+            h.update(f.encode())
             with open(p, "rb") as fh:
                 h.update(fh.read())
     h.update(" ".join(spec["defines"] + DEVICE_FLAGS + HOST_FLAGS).encode())
@@ -162,13 +164,15 @@ def build(name: str, verbose: bool = True, jobs: int = 0) -> str:
 
 
 def ensure(name: str, verbose: bool = True) -> str:
-    """Path of a built library, building it first only if none is there."""
+    """Path of a library that was built from the sources as they are now: a library whose
+    stamp matches is used, anything else (none there, or one older than its sources) is
+    built first.  A stale library is never loaded: without hipcc this raises."""
     out = lib_path(name)
-    if os.path.isfile(out):
-        if not is_current(name) and verbose:
-            print(f"[zse_amd] note: {out} is older than its sources; using it as it is "
-                  f"(rebuild with `python -m zse_amd build`)", file=sys.stderr, flush=True)
+    if os.path.isfile(out) and is_current(name):
         return out
+    if os.path.isfile(out) and verbose:
+        print(f"[zse_amd] {out} does not match its sources; building it again", file=sys.stderr,
+              flush=True)
     return build(name, verbose=verbose)
 
 
