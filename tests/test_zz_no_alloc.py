@@ -1,0 +1,119 @@
+"""The matrix product that allocates nothing (zk_gemm_bf16_static), called through ctypes as a
+caller outside the package would, against zk_gemm_bf16 with its workspace: the same bits, on
+two calls in a row of which the second is smaller, with the array's old contents in the way."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+VP, I, F = C.c_void_p, C.c_int, C.c_float
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from zse_amd.runtime.device import Runtime
+    return Runtime.get()
+
+
+@pytest.fixture(scope="module")
+def dll(rt):
+    from zse_amd.runtime import build
+    rt.kernels("bfloat16")                       # makes sure the library is built
+    lib = C.CDLL(build.lib_path("kernels_bf16"))
+    lib.zk_last_error.restype = C.c_char_p
+    lib.zk_gemm_bf16_static_bytes.restype = C.c_size_t
+    lib.zk_gemm_bf16_static_bytes.argtypes = []
+    lib.zk_gemm_bf16_static_init.restype = I
+    lib.zk_gemm_bf16_static_init.argtypes = []
+    lib.zk_gemm_bf16_static.restype = I
+    lib.zk_gemm_bf16_static.argtypes = [VP, I, VP, VP, I, I, I, I, I, I, F, I, VP]
+    lib.zk_gemm_bf16.restype = I
+    lib.zk_gemm_bf16.argtypes = [VP, I, VP, VP, I, I, I, I, I, I, F, I, VP, C.c_size_t, C.POINTER(I), VP]
+    lib.zk_strip_layout.restype = I
+    lib.zk_strip_layout.argtypes = [VP, VP, I, I, VP]
+    return lib
+
+
+def bf16_bits(x):
+    from zse_amd.weights.safetensors import f32_to_bf16_bits
+    return f32_to_bf16_bits(np.ascontiguousarray(x, np.float32))
+
+
+def operands(rt, dll, M, N, K, seed, strip, gated=False):
+    rng = np.random.default_rng(seed)
+    rows = 2 * N if gated else N
+    A = rt.upload(bf16_bits(rng.normal(size=(M, K))), "bfloat16")
+    W = rt.upload(bf16_bits(rng.normal(size=(rows, K)) * (0.3 if gated else 1.0)), "bfloat16")
+    if strip:
+        Ws = rt.empty(((rows + 15) // 16 * 16, K), "bfloat16")
+        assert dll.zk_strip_layout(W.ptr, Ws.ptr, rows, K, rt.stream) == 0, dll.zk_last_error()
+        rt.sync()
+        W = Ws
+    return A, W
+
+
+def both(rt, dll, ws, M, N, K, seed, strip=1, epi=0, f32_out=0):
+    """(bits from the static entry point, bits from zk_gemm_bf16 with its workspace)."""
+    A, W = operands(rt, dll, M, N, K, seed, strip, gated=epi >= 2)
+    dt = "float32" if f32_out else "bfloat16"
+    got, want = rt.zeros((M, N), dt), rt.zeros((M, N), dt)
+    rc = dll.zk_gemm_bf16_static(A.ptr, K, W.ptr, got.ptr, N, f32_out, M, N, K, epi, 0.0, strip, rt.stream)
+    assert rc == 0, dll.zk_last_error().decode()
+    rc = dll.zk_gemm_bf16(A.ptr, K, W.ptr, want.ptr, N, f32_out, M, N, K, epi, 0.0, strip, ws.ptr, ws.nbytes,
+                          None, rt.stream)
+    assert rc == 0, dll.zk_last_error().decode()
+    g, w = rt.download(got), rt.download(want)
+    assert np.abs(w.astype(np.float64)).max() > 0
+    return g, w
+
+
+def ranges_of(rt, dll, ws, M, N, K):
+    """Into how many ranges zk_gemm_bf16 splits K for this shape (0: not at all)."""
+    A, W = operands(rt, dll, M, N, K, 0, 1)
+    out = rt.zeros((M, N), "bfloat16")
+    parts = I(0)
+    rc = dll.zk_gemm_bf16(A.ptr, K, W.ptr, out.ptr, N, 0, M, N, K, 0, 0.0, 1, ws.ptr, ws.nbytes,
+                          C.byref(parts), rt.stream)
+    assert rc == 0, dll.zk_last_error().decode()
+    rt.sync()
+    return parts.value
+
+
+def test_static_product_equals_the_one_with_a_workspace(rt, dll):
+    assert dll.zk_gemm_bf16_static_bytes() == 8 << 20
+    assert dll.zk_gemm_bf16_static_init() == 0, dll.zk_last_error().decode()
+    assert dll.zk_gemm_bf16_static_init() == 0           # a second set-up call changes nothing
+    ws = rt.zeros((rt.kernels("bfloat16").zk_gemm_bf16_workspace() // 4,), "float32")
+    # 40 rows, N = 2304: 36 column blocks, so K is split into 7 ranges whose partial sums
+    # (7 planes of [40, 2304] floats, 2.6 MB) go through the static array
+    g, w = both(rt, dll, ws, 40, 2304, 2304, seed=1)
+    assert np.array_equal(g, w)
+    assert ranges_of(rt, dll, ws, 40, 2304, 2304) == 7     # the shape does go through the scratch memory
+    # the second call is smaller: other plane sizes, over what the first call left behind
+    g, w = both(rt, dll, ws, 24, 1152, 1024, seed=2)
+    assert np.array_equal(g, w)
+    # a third, larger again and gated (two planes a range), float output
+    g, w = both(rt, dll, ws, 64, 1024, 2048, seed=3, epi=2, f32_out=1)
+    assert np.array_equal(g, w)
+    # many rows, few tiles and a long K: the tile kernel splits K and joins through the array
+    g, w = both(rt, dll, ws, 100, 200, 2048, seed=4, strip=0, f32_out=1)
+    assert np.array_equal(g, w)
+    # few rows without a split: the array is not touched, the result is still the same
+    g, w = both(rt, dll, ws, 8, 2304, 2048, seed=5)
+    assert np.array_equal(g, w)
+
+
+def test_static_product_refuses_what_does_not_fit(rt, dll):
+    # 1024 rows, N = 1024, K = 16384: 64 tiles of 128 x 128 split K into 4 ranges, 16 MB of
+    # partial sums; the array holds 8 MB, so the call is refused and nothing is launched
+    M, N, K = 1024, 1024, 16384
+    A = rt.zeros((M, K), "bfloat16")
+    W = rt.zeros((N, K), "bfloat16")
+    out = rt.zeros((M, N), "bfloat16")
+    rc = dll.zk_gemm_bf16_static(A.ptr, K, W.ptr, out.ptr, N, 0, M, N, K, 0, 0.0, 0, rt.stream)
+    assert rc != 0
+    msg = dll.zk_last_error().decode()
+    assert "static scratch array holds 8388608" in msg and "need" in msg
+    rt.sync()

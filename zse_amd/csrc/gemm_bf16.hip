@@ -20,6 +20,26 @@
 // (orchestrator/kernels.py:1075-1126, 2077-2107), gate and up separate
 // (orchestrator/model_runner.py:1270-1275).
 #include "common.h"
+#include "gemm_bf16_static.h"
+
+#include <mutex>
+
+// Where a product that splits K over blocks leaves its partial sums.  ``strict``: the split is
+// chosen as for the standard workspace (so that the bits do not depend on who brought the
+// memory) and refused, not narrowed, when ``bytes`` cannot hold it.
+#define ZK_GEMM_WORKSPACE_BYTES ((size_t)32 << 20)
+struct GemmWorkspace {
+  void* ptr;
+  size_t bytes;
+  bool strict;
+  size_t split_bytes() const { return strict ? ZK_GEMM_WORKSPACE_BYTES : bytes; }
+  int too_small(size_t need) const {
+    static thread_local char msg[200];
+    snprintf(msg, sizeof msg, "zk_gemm_bf16_static: this shape's partial sums need %zu bytes, the "
+             "static scratch array holds %zu", need, bytes);
+    return zk_fail(msg);
+  }
+};
 
 #if ZSE_ACT_BF16
 
@@ -534,7 +554,7 @@ __global__ __launch_bounds__(256) void gemm_tile_join_kernel(
 
 template <int WMT, int NWM, int NWN, bool GATED, bool EXACT>
 static int launch_tile(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M, int N,
-                       int K, int epi, float cap, int w_strip, void* ws, size_t ws_bytes, int ksplit,
+                       int K, int epi, float cap, int w_strip, const GemmWorkspace& wsp, int ksplit,
                        hipStream_t s) {
   constexpr int BM = 32 * WMT * NWM, BN = 64 * NWN;
   constexpr int ncols = GATED ? BN / 2 : BN;
@@ -551,8 +571,10 @@ static int launch_tile(const void* A, int lda, const void* W, void* C, int ldc, 
   ZK_REQUIRE((long long)tiles_m * tiles_n < 2147483647LL, "zk_gemm_bf16: too many tiles");
   // K split over blockIdx.y only as far as the partial sums fit the workspace
   const size_t per_range = (size_t)tiles_m * tiles_n * BM * BN * sizeof(float);
+  void* ws = wsp.ptr;
   if (ws == nullptr || (uintptr_t)ws % 64 != 0) ksplit = 1;
-  while (ksplit > 1 && per_range * ksplit > ws_bytes) ksplit--;
+  while (ksplit > 1 && per_range * ksplit > wsp.split_bytes()) ksplit--;
+  if (ksplit > 1 && per_range * ksplit > wsp.bytes) return wsp.too_small(per_range * ksplit);
   gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT><<<dim3(tiles_m * tiles_n, ksplit), 64 * NWM * NWN, lds, s>>>(
       (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, tiles_m, tiles_n, w_strip,
       (f32x16*)ws, ksplit);
@@ -745,7 +767,7 @@ __global__ __launch_bounds__(256) void gemm_join_kernel(const float* __restrict_
 
 template <bool GATED>
 static int launch_mid(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M, int N,
-                      int K, int epi, float cap, void* ws, size_t ws_bytes, int* parts, hipStream_t s) {
+                      int K, int epi, float cap, const GemmWorkspace& wsp, int* parts, hipStream_t s) {
   const int mt = (M + 15) / 16;
   const int npad = (N + 15) / 16 * 16;
   const int cblocks = ((N + 15) / 16 + 3) / 4;
@@ -755,8 +777,10 @@ static int launch_mid(const void* A, int lda, const void* W, void* C, int ldc, i
   if (ksplit > K / 32 / GM_STEPS) ksplit = K / 32 / GM_STEPS;
   if (ksplit < 1) ksplit = 1;
   const size_t per_range = (size_t)(GATED ? 2 : 1) * M * npad * sizeof(float);
+  void* ws = wsp.ptr;
   if (ws == nullptr || (uintptr_t)ws % 16 != 0) ksplit = 1;
-  while (ksplit > 1 && ksplit * per_range > ws_bytes) ksplit--;
+  while (ksplit > 1 && ksplit * per_range > wsp.split_bytes()) ksplit--;
+  if (ksplit > 1 && ksplit * per_range > wsp.bytes) return wsp.too_small(ksplit * per_range);
   float* partials = (float*)ws;
   dim3 grid(cblocks, ksplit);
 #define ZK_MID(MT_)                                                                                   \
@@ -870,11 +894,11 @@ extern "C" int zk_strip_layout(const void* src, void* dst, int N, int K, void* s
 // for their number.  0 comes back when the result is in C as usual; P > 0 when C was not
 // written and the workspace starts with P planes of [M, N] floats, to be added in order and
 // rounded to 16 bits (zk_norm_add_norm reads them so), before the next product overwrites them.
-extern "C" size_t zk_gemm_bf16_workspace() { return (size_t)32 << 20; }
+extern "C" size_t zk_gemm_bf16_workspace() { return ZK_GEMM_WORKSPACE_BYTES; }
 
-extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
-                            int M, int N, int K, int epi, float cap, int w_strip, void* ws,
-                            size_t ws_bytes, int* parts, void* stream) {
+static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
+                         int M, int N, int K, int epi, float cap, int w_strip, const GemmWorkspace& wsp,
+                         int* parts, void* stream) {
   ZK_REQUIRE(M >= 0 && N > 0 && K > 0, "zk_gemm_bf16: bad sizes");
   ZK_REQUIRE(K % 8 == 0 && lda % 8 == 0, "zk_gemm_bf16: K and lda must be multiples of 8");
   ZK_REQUIRE(lda >= K && ldc >= N, "zk_gemm_bf16: leading dimensions too small");
@@ -887,8 +911,8 @@ extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int 
   if (M == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (M > 16 && M <= 64 && w_strip) {
-    return gated ? launch_mid<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, ws, ws_bytes, parts, s)
-                 : launch_mid<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, ws, ws_bytes, parts, s);
+    return gated ? launch_mid<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, wsp, parts, s)
+                 : launch_mid<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, wsp, parts, s);
   }
   if (M <= 64) {
     return gated ? launch_skinny<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s)
@@ -920,7 +944,7 @@ extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int 
   const bool low = !wide && M > 64 && nb_small * ksplit <= 128;
   if (low) ksplit = ranges((long)((M + 63) / 64) * (nb_small / tiles_m));
 #define ZK_TILE_(W_, M_, N_, G_, E_) \
-  launch_tile<W_, M_, N_, G_, E_>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, ws, ws_bytes, ksplit, s)
+  launch_tile<W_, M_, N_, G_, E_>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, wsp, ksplit, s)
 #define ZK_TILE(W_, M_, N_)                                                                            \
   (gated ? (exact ? ZK_TILE_(W_, M_, N_, true, true) : ZK_TILE_(W_, M_, N_, true, false))             \
          : (exact ? ZK_TILE_(W_, M_, N_, false, true) : ZK_TILE_(W_, M_, N_, false, false)))
@@ -929,6 +953,63 @@ extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int 
   return ZK_TILE(2, 2, 2);
 #undef ZK_TILE
 #undef ZK_TILE_
+}
+
+extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
+                            int M, int N, int K, int epi, float cap, int w_strip, void* ws,
+                            size_t ws_bytes, int* parts, void* stream) {
+  return gemm_bf16_run(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, GemmWorkspace{ws, ws_bytes, false},
+                       parts, stream);
+}
+
+// ---- the same product for callers that cannot allocate (declared in gemm_bf16_static.h)
+//
+// The partial sums of a product that splits K go to a statically allocated array instead of a
+// workspace the caller brings.  Every GPU holds its own copy of the array at its own address;
+// host code never uses the array's name as an address, only the pointer that
+// hipGetSymbolAddress gave for the device that is current.
+static __device__ __align__(256) unsigned char scratch[ZK_GEMM_STATIC_SCRATCH_BYTES];
+
+#define ZK_MAX_DEVICES 64
+static void* scratch_of_device[ZK_MAX_DEVICES];     // null until the device's set-up has run
+static std::mutex scratch_mutex;
+
+// The array's address on the current device, asked for once per device.
+static int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return zk_fail("zk_gemm_bf16_static: no current device");
+  ZK_REQUIRE(dev >= 0 && dev < ZK_MAX_DEVICES, "zk_gemm_bf16_static: device index out of range");
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_of_device[dev] == nullptr) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      (void)hipGetLastError();
+      return zk_fail("zk_gemm_bf16_static: hipGetSymbolAddress of the scratch array failed");
+    }
+    scratch_of_device[dev] = ptr;
+  }
+  *out = scratch_of_device[dev];
+  return 0;
+}
+
+extern "C" size_t zk_gemm_bf16_static_bytes() { return ZK_GEMM_STATIC_SCRATCH_BYTES; }
+
+extern "C" int zk_gemm_bf16_static_init() {
+  void* ptr = nullptr;
+  return static_scratch(&ptr);
+}
+
+extern "C" int zk_gemm_bf16_static(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
+                                   int M, int N, int K, int epi, float cap, int w_strip, void* stream) {
+  void* ptr = nullptr;
+  if (int rc = static_scratch(&ptr)) return rc;
+  // strict: K is split exactly as zk_gemm_bf16 splits it with its standard workspace, so the
+  // results have the same bits; a split whose partial sums do not fit the array is refused.
+  // Nothing in the array has to start at zero: each range's plane is written in full by the
+  // product kernel before the joining kernel of the same call reads it.
+  return gemm_bf16_run(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip,
+                       GemmWorkspace{ptr, ZK_GEMM_STATIC_SCRATCH_BYTES, true}, nullptr, stream);
 }
 
 #endif  // ZSE_ACT_BF16

@@ -161,6 +161,7 @@ KERNEL_SIGNATURES = {
 # present only in the bf16 library
 BF16_KERNEL_SIGNATURES = {
     "zk_gemm_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, C.c_size_t, C.POINTER(C.c_int), _VP],
+    "zk_gemm_bf16_static": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
     "zk_strip_layout": [_VP, _VP, _I, _I, _VP],
     "zk_qkv_rope_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "zk_attention_bf16": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
