@@ -53,14 +53,15 @@ def make_runner(folder, dtype, **kw):
     return StepRunner(model, rt, dtype, **kw)
 
 
-def run_steps(runner, streams, steps):
+def run_steps(runner, streams, steps, observe=None):
     """``streams``: {req: tokens}; ``steps``: list of (entries, ends) with entries a list
     of (req, n).  Feeds each request's next n tokens, wants every logit.  Returns
-    {req: [rows in position order]}."""
+    {req: [rows in position order]}.  ``observe(step index)`` is called after each step
+    has run, before the requests it ends give their pages back."""
     from zse_amd.engine.runner import StepEntry
     fed = {r: 0 for r in streams}
     rows = {r: [] for r in streams}
-    for entries, ends in steps:
+    for step_index, (entries, ends) in enumerate(steps):
         es = []
         for r, n in entries:
             es.append(StepEntry(r, streams[r][fed[r]:fed[r] + n], list(range(n))))
@@ -70,6 +71,8 @@ def run_steps(runner, streams, steps):
             rows[r].extend(z[at:at + n])
             at += n
             fed[r] += n
+        if observe is not None:
+            observe(step_index)
         for r in ends:
             runner.finish(r)
         runner.manager.check()
@@ -103,16 +106,21 @@ def chunked_steps(streams, sizes=(7, 2, 5, 3, 2, 11, 2, 4)):
     return steps
 
 
-def mixed_steps(streams, seed=0, max_live=4, decode_tail=12, chunk_choices=(2, 3, 5, 9)):
+def mixed_steps(streams, seed=0, max_live=4, decode_tail=12, chunk_choices=(2, 3, 5, 9), room=None, page=1):
     """Up to ``max_live`` requests at a time: prompt portions of some beside single
     tokens of others (a request decodes one by one over its last ``decode_tail``
-    tokens); requests enter as others leave; some sit a step out."""
+    tokens); requests enter as others leave; some sit a step out.  ``room``: pages of
+    ``page`` tokens the pool has; a request enters only while the live requests, each at
+    its full length, and it fit together."""
     rng = np.random.default_rng(seed)
     waiting = list(streams)
     live, fed = [], {}
     steps = []
+    pages_of = lambda r: -(-len(streams[r]) // page)
     while waiting or live:
         while waiting and len(live) < max_live:
+            if room is not None and sum(pages_of(r) for r in live) + pages_of(waiting[0]) > room:
+                break
             r = waiting.pop(0)
             live.append(r)
             fed[r] = 0

@@ -159,3 +159,30 @@ def test_random_orders_keep_every_invariant(seed):
         m.release(r)
     m.check()
     assert all(p.free_pages == p.num_pages for p in m.pools) and m.slots.free_slots == 4
+
+
+def test_attention_workspace_follows_the_models_limits():
+    """The split attention's workspace is what its kernel asks for at the runner's limits:
+    requests x heads x chunks of 64 keys x (head_dim + 2) floats.  At 64 requests of 8192
+    tokens the two larger models need more than the 128 MB a fixed buffer once gave them."""
+    from zse_amd.config import AttentionSpec, RotarySpec
+    from zse_amd.parts import build_part
+    from zse_amd.runtime import build
+    from zse_amd.runtime.device import KernelLibrary
+    try:
+        k = KernelLibrary(build.ensure("kernels_bf16", verbose=False), "bfloat16")
+    except build.BuildError as e:
+        pytest.skip(f"the kernel library cannot be built here: {e}")
+    for nh, nkv, hd, want in [(8, 4, 256, 67633152), (16, 8, 256, 135266304), (32, 16, 128, 136314880)]:
+        spec = AttentionSpec(1024, nh, nkv, hd, hd ** -0.5, 50.0, None, RotarySpec(hd, hd, 1e4),
+                             {r: r for r in "qkvo"})
+        part = build_part("mixer", spec)
+        need = part.prepare(k, "bfloat16", 64, 8192, 16)
+        assert need == want == 64 * nh * 128 * (hd + 2) * 4
+        assert part.decode_chunk == 64
+        assert part.prepare(k, "bfloat16", 1, 4096, 16) == nh * 64 * (hd + 2) * 4
+        assert part.decode_chunk == (32 if nkv * 64 <= 512 else 64)      # one request: finer cuts while waves are few
+        assert part.prepare(k, "float32", 64, 8192, 16) == 0           # the plain kernel needs none
+    # a context the decode kernel cannot join is refused when the runner is made, with the numbers
+    with pytest.raises(ValueError, match="longest context"):
+        part.prepare(k, "bfloat16", 64, 300000, 16)

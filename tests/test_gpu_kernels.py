@@ -360,20 +360,133 @@ def test_attention_over_pages(rt, kernel, case):
     POS, REQ = rt.upload(np.array(tok_pos, np.int32)), rt.upload(np.array(tok_req, np.int32))
     qs = np.concatenate([[0], np.cumsum([n for _, n in reqs])]).astype(np.int32)
     QS, CL = rt.upload(qs), rt.upload(np.array(total, np.int32))
-    OUT = rt.zeros((T, nh * hd), dtype)
-    if kernel == "mfma":
-        n_multi = sum(1 for _, n in reqs if n > 1)
-        ws = rt.zeros((max(1, k.zk_attention_bf16_workspace(R, nh, hd, max(total)) // 4),), "float32")
-        k.zk_attention_bf16(Q.ptr, nh * hd, KC.ptr, VC.ptr, TBL.ptr, max_blocks, QS.ptr, CL.ptr, OUT.ptr,
-                            R, n_multi, max(n for _, n in reqs), max(total), nh, nkv, hd, bs, scale,
-                            c["cap"], c["window"], ws.ptr, ws.nbytes, rt.stream)
-    else:
-        k.zk_attention_plain(Q.ptr, nh * hd, KC.ptr, VC.ptr, TBL.ptr, max_blocks, REQ.ptr, POS.ptr, OUT.ptr,
-                             T, nh, nkv, hd, bs, scale, c["cap"], c["window"], 1 if vt else 0, rt.stream)
-    got = rt.download_f32(OUT).reshape(T, nh, hd)
     tol = 2e-5 if dtype == "float32" else 0.02
-    err = np.abs(got - want)
-    assert err.max() < tol, f"max error {err.max()} at token {np.unravel_index(err.argmax(), err.shape)}"
+    outs = []
+    for chunk in ((64, 32) if kernel == "mfma" else (0,)):      # both cuts of the decoded tokens' keys
+        OUT = rt.zeros((T, nh * hd), dtype)
+        if kernel == "mfma":
+            n_multi = sum(1 for _, n in reqs if n > 1)
+            # more context allowed than any request has, as in a captured step: more chunks than keys
+            max_ctx = max(total) + 200
+            ws = rt.zeros((max(1, k.zk_attention_bf16_workspace(R, nh, hd, max_ctx) // 4),), "float32")
+            k.zk_attention_bf16(Q.ptr, nh * hd, KC.ptr, VC.ptr, TBL.ptr, max_blocks, QS.ptr, CL.ptr, OUT.ptr,
+                                R, n_multi, max(n for _, n in reqs), max_ctx, nh, nkv, hd, bs, scale,
+                                c["cap"], c["window"], chunk, ws.ptr, ws.nbytes, rt.stream)
+        else:
+            k.zk_attention_plain(Q.ptr, nh * hd, KC.ptr, VC.ptr, TBL.ptr, max_blocks, REQ.ptr, POS.ptr, OUT.ptr,
+                                 T, nh, nkv, hd, bs, scale, c["cap"], c["window"], 1 if vt else 0, rt.stream)
+        got = rt.download_f32(OUT).reshape(T, nh, hd)
+        err = np.abs(got - want)
+        assert err.max() < tol, (f"chunk {chunk}: max error {err.max()} at token "
+                                 f"{np.unravel_index(err.argmax(), err.shape)}")
+        outs.append(got)
+
+
+def run_attention(rt, kernel, q, kk, vv, past, nh, nkv, hd, bs, scale, cap, window, chunk=64, max_ctx=None):
+    """One request holding ``past`` cached tokens brings the rest of ``kk``/``vv`` [ctx, nkv, hd]
+    with queries ``q`` [n, nh, hd]; pages are laid out in order.  Returns [n, nh, hd]."""
+    dtype = "float32" if kernel == "plain_f32" else "bfloat16"
+    k = rt.kernels(dtype)
+    vt = kernel == "mfma"
+    ctx, n = kk.shape[0], q.shape[0]
+    assert past + n == ctx
+    nblk = -(-ctx // bs)
+    kc = np.zeros((nblk, nkv, bs, hd), np.float32)
+    vc = np.zeros((nblk, nkv, hd, bs) if vt else (nblk, nkv, bs, hd), np.float32)
+    for j in range(nblk):
+        bk, bv = kk[j * bs:(j + 1) * bs], vv[j * bs:(j + 1) * bs]
+        kc[j, :, :len(bk)] = bk.transpose(1, 0, 2)
+        if vt:
+            vc[j, :, :, :len(bv)] = bv.transpose(1, 2, 0)
+        else:
+            vc[j, :, :len(bv)] = bv.transpose(1, 0, 2)
+    Q, KC, VC = up(rt, q.reshape(n, nh * hd), dtype), up(rt, kc, dtype), up(rt, vc, dtype)
+    TBL = rt.upload(np.arange(nblk, dtype=np.int32).reshape(1, nblk))
+    QS, CL = rt.upload(np.array([0, n], np.int32)), rt.upload(np.array([ctx], np.int32))
+    POS, REQ = rt.upload(np.arange(past, ctx, dtype=np.int32)), rt.upload(np.zeros(n, np.int32))
+    OUT = rt.zeros((n, nh * hd), dtype)
+    if kernel == "mfma":
+        max_ctx = max_ctx or ctx
+        ws = rt.zeros((max(1, k.zk_attention_bf16_workspace(1, nh, hd, max_ctx) // 4),), "float32")
+        k.zk_attention_bf16(Q.ptr, nh * hd, KC.ptr, VC.ptr, TBL.ptr, nblk, QS.ptr, CL.ptr, OUT.ptr, 1,
+                            1 if n > 1 else 0, n, max_ctx, nh, nkv, hd, bs, scale, cap or 0.0, window or 0,
+                            chunk, ws.ptr, ws.nbytes, rt.stream)
+    else:
+        k.zk_attention_plain(Q.ptr, nh * hd, KC.ptr, VC.ptr, TBL.ptr, nblk, REQ.ptr, POS.ptr, OUT.ptr, n, nh,
+                             nkv, hd, bs, scale, cap or 0.0, window or 0, 0, rt.stream)
+    return rt.download_f32(OUT).reshape(n, nh, hd)
+
+
+@pytest.mark.parametrize("kernel", ["plain_f32", "plain_bf16", "mfma"])
+def test_attention_scales_then_caps_then_masks(rt, kernel):
+    # q1.k0 = 1e4, q1.k1 = 0, q0.k0 = -1e4, v0 = 1, v1 = 0, scale 0.01, cap 50 (all exact in bf16):
+    # right order o1 = 1.000 and o0 = 1; the cap before the scale gives o1 = 0.622; the mask
+    # before the cap lets the hidden key 1 into o0 = 0.858
+    from test_plain import cap_order_vectors
+    q, kk, vv, scale, cap = cap_order_vectors(16)
+    tol = 1e-5 if kernel == "plain_f32" else 4e-3
+    # both tokens as one portion
+    o = run_attention(rt, kernel, q, kk, vv, 0, 1, 1, 16, 4, scale, cap, None)
+    assert abs(o[1, 0, 0] - 1.0) < tol and abs(o[0, 0, 0] - 1.0) < tol, o[:, 0, 0]
+    # each as a decoded token: query 0 with key 1 lying in the cache past its context, query 1
+    for chunk in (64, 32):
+        o0 = run_attention(rt, kernel, q[:1], kk[:1], vv[:1], 0, 1, 1, 16, 4, scale, cap, None, chunk)
+        o1 = run_attention(rt, kernel, q[1:], kk, vv, 1, 1, 1, 16, 4, scale, cap, None, chunk)
+        assert abs(o0[0, 0, 0] - 1.0) < tol and abs(o1[0, 0, 0] - 1.0) < tol, (o0[0, 0, 0], o1[0, 0, 0])
+    # a softer pair where the cap decides the weights: scores 10 and 9 capped at 5 are nearly a tie
+    k2 = np.stack([kk[0], kk[0] * 0.9]); v2 = np.stack([vv[0], vv[1]])
+    want = 1 / (1 + math.exp(5 * math.tanh(1.8) - 5 * math.tanh(2.0)))      # 0.5215; uncapped: 0.731
+    o = run_attention(rt, kernel, q / 10, k2, v2, 0, 1, 1, 16, 4, scale, 5.0, None)
+    assert abs(o[1, 0, 0] - want) < max(tol, 2e-3)
+
+
+def test_decode_attention_at_a_large_models_limits(rt):
+    """64 decoded tokens at the head geometry of the largest model (32 heads, 16 KV heads of 128)
+    in a step that allows 8192 tokens of context while the requests hold few: the workspace is
+    what the kernel says it needs for these limits (136 MB), and the result is the plain kernel's."""
+    k = rt.kernels("bfloat16")
+    nh, nkv, hd, bs, R, max_ctx = 32, 16, 128, 16, 64, 8192
+    need = k.zk_attention_bf16_workspace(R, nh, hd, max_ctx)
+    assert need == R * nh * (max_ctx // 64) * (hd + 2) * 4 == 136314880
+    rng = np.random.default_rng(5)
+    ctxs = rng.integers(1, 300, R)
+    ctxs[0], ctxs[1], ctxs[2] = 1, 64, 257
+    max_blocks = max_ctx // bs
+    pages = int(sum(-(-c // bs) for c in ctxs)) + 1
+    kc = bf16(rng.normal(size=(pages, nkv, bs, hd)))
+    v = bf16(rng.normal(size=(pages, nkv, bs, hd)))
+    vt = np.ascontiguousarray(v.transpose(0, 1, 3, 2))
+    table = np.full((R, max_blocks), -1, np.int32)
+    at = 1                                                  # page 0 belongs to nobody
+    for r, c in enumerate(ctxs):
+        nb = -(-int(c) // bs)
+        table[r, :nb] = np.arange(at, at + nb)
+        at += nb
+    q = bf16(rng.normal(size=(R, nh * hd)))
+    Q, KC, V, VT = up(rt, q, "bfloat16"), up(rt, kc, "bfloat16"), up(rt, v, "bfloat16"), up(rt, vt, "bfloat16")
+    TBL = rt.upload(table)
+    QS, CL = rt.upload(np.arange(R + 1, dtype=np.int32)), rt.upload(ctxs.astype(np.int32))
+    POS, REQ = rt.upload((ctxs - 1).astype(np.int32)), rt.upload(np.arange(R, dtype=np.int32))
+    want_t = rt.zeros((R, nh * hd), "bfloat16")
+    k.zk_attention_plain(Q.ptr, nh * hd, KC.ptr, V.ptr, TBL.ptr, max_blocks, REQ.ptr, POS.ptr, want_t.ptr, R,
+                         nh, nkv, hd, bs, 144 ** -0.5, 50.0, 0, 0, rt.stream)
+    want = rt.download_f32(want_t)
+    ws = rt.zeros((need // 4,), "float32")
+    for chunk in (64, 32):
+        out = rt.zeros((R, nh * hd), "bfloat16")
+        k.zk_attention_bf16(Q.ptr, nh * hd, KC.ptr, VT.ptr, TBL.ptr, max_blocks, QS.ptr, CL.ptr, out.ptr, R, 0,
+                            1, max_ctx, nh, nkv, hd, bs, 144 ** -0.5, 50.0, 0, chunk, ws.ptr, ws.nbytes, rt.stream)
+        assert np.abs(rt.download_f32(out) - want).max() < 0.02
+    # one byte less and the call is refused before anything is launched
+    from zse_amd.runtime.device import DeviceError
+    with pytest.raises(DeviceError, match="workspace too small"):
+        k.zk_attention_bf16(Q.ptr, nh * hd, KC.ptr, VT.ptr, TBL.ptr, max_blocks, QS.ptr, CL.ptr, out.ptr, R, 0,
+                            1, max_ctx, nh, nkv, hd, bs, 144 ** -0.5, 50.0, 0, 64, ws.ptr, ws.nbytes - 4, rt.stream)
+    # a context beyond what the joining kernel can weigh is refused with its own message
+    too_long = int(k.zk_attention_bf16_max_context(nh, nkv, hd, 64)) + 1
+    with pytest.raises(DeviceError, match="context too long"):
+        k.zk_attention_bf16(Q.ptr, nh * hd, KC.ptr, VT.ptr, TBL.ptr, max_blocks, QS.ptr, CL.ptr, out.ptr, R, 0,
+                            1, too_long, nh, nkv, hd, bs, 144 ** -0.5, 50.0, 0, 64, ws.ptr, 1 << 40, rt.stream)
 
 
 # ------------------------------------------------------------------ row-wise kernels

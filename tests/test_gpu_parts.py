@@ -162,55 +162,12 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(rt):
     """A mixer the framework has never heard of: out_t = s_t W^T with s_t = a * s_(t-1) + x_t kept per
     request in its state slot.  Its architecture is registered here, built through the registry and
     stepped in portions and in mixed batches; the cut must not change the result."""
-    from dataclasses import dataclass
-    from zse_amd.config import (Architecture, BlockSpec, EmbeddingSpec, GatedMLPSpec, HeadSpec, LayerCall,
-                                ModelPlan, NormSpec, register_architecture, unregister_architecture)
+    from zse_amd.config import BlockSpec, EmbeddingSpec, GatedMLPSpec, HeadSpec, LayerCall, ModelPlan, NormSpec
     from zse_amd.engine.loading import random_model
     from zse_amd.engine.runner import StepEntry, StepRunner
-    from zse_amd.parts import Part, StateNeed, TensorReq, register_part, unregister_part
-    from zse_amd.parts.ops import linear
+    from toy_state import DecaySpec, toy_architecture
 
     H, V, I, L, A = 64, 200, 96, 2, 0.75
-
-    @dataclass(frozen=True)
-    class DecaySpec:
-        hidden_size: int
-        decay: float
-        weight: str
-        kind: str = "toy_decay"
-
-    class DecayMixer(Part):
-        def __init__(self, spec):
-            self.spec, self.w = spec, None
-
-        def tensor_reqs(self):
-            return [TensorReq(self.spec.weight, (self.spec.hidden_size, self.spec.hidden_size))]
-
-        def load(self, weights, rt_, dtype):
-            self.w = weights.matrix([self.spec.weight])
-
-        def cache_need(self):
-            return StateNeed(self.spec.hidden_size * 4)
-
-        def forward(self, ctx, x, cache):
-            # the recurrence runs on the host here (a toy): rows in, rows out, state in the slot
-            xs = ctx.rt.download_f32(x)
-            words = ctx.slot_bytes // 4
-            state = ctx.rt.download(ctx.state)
-            o0, n_w = cache.state_offset // 4, cache.state_bytes // 4
-            out = np.empty_like(xs)
-            t = 0
-            for _, slot, _, n in ctx.entries:
-                s = state[slot, o0:o0 + n_w].copy()
-                for i in range(n):
-                    s = np.float32(self.spec.decay) * s + xs[t + i]
-                    out[t + i] = s
-                state[slot, o0:o0 + n_w] = s
-                t += n
-            ctx.rt.copy_h2d(ctx.state.ptr, state)
-            y = ctx.alloc(x.shape)
-            ctx.rt.copy_h2d(y.ptr, out)
-            return linear(ctx, y, self.w, ctx.alloc(x.shape))
 
     def plan_of(cfg):
         norm = lambda n: NormSpec(H, 1e-6, False, n)
@@ -220,9 +177,7 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(rt):
         return ModelPlan("ToyDecayLM", H, V, 512, EmbeddingSpec(V, H, 1.0, "emb"), layers,
                          tuple(LayerCall(l) for l in range(L)), norm("final"), HeadSpec(V, H, None, "emb"))
 
-    register_part("mixer", "toy_decay", DecayMixer)
-    register_architecture(Architecture("ToyDecayLM", lambda d: d, plan_of))
-    try:
+    with toy_architecture("ToyDecayLM", plan_of):
         model = random_model({"architectures": ["ToyDecayLM"]}, "float32", seed=4, std=0.1, gain_std=0.1, rt=rt)
         runner = StepRunner(model, rt, "float32", page_size=4, cache_tokens=64, max_seqs=3, max_batch_tokens=64,
                             max_model_len=128, use_graphs=False)
@@ -257,6 +212,57 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(rt):
         assert np.array_equal(again, whole_a)
         # and the state really carries: against the recurrence done by hand for layer 0's mixer input
         assert not np.allclose(whole_a[5], runner.step([StepEntry("d", a[5:6], [0])])[0])
-    finally:
-        unregister_part("mixer", "toy_decay")
-        unregister_architecture("ToyDecayLM")
+        assert not runner.graph_safe          # the toy reads the step's description on the host
+
+
+def test_toy_mixer_with_state_through_the_engine(rt):
+    """The same toy mixer behind the scheduler: layer 0 keeps its recurrence in the request's
+    state slot, layer 1 is the framework's attention over pages.  Six requests share two slots
+    and a pool so small that requests are preempted and computed again; every slot a request
+    gets, first or again, must start from zero, so each request's tokens equal its run alone."""
+    from zse_amd.config import (AttentionSpec, BlockSpec, EmbeddingSpec, GatedMLPSpec, HeadSpec, LayerCall,
+                                ModelPlan, NormSpec, RotarySpec)
+    from zse_amd.engine.engine import Engine
+    from zse_amd.engine.loading import random_model
+    from zse_amd.sampling import SamplingParams
+    from toy_state import DecaySpec, toy_architecture
+
+    H, V, I, nh, nkv, hd = 64, 200, 96, 4, 2, 16
+
+    def plan_of(cfg):
+        norm = lambda n: NormSpec(H, 1e-6, False, n)
+        ffn = lambda l: GatedMLPSpec(H, I, "silu", {r: f"l{l}.ffn.{r}" for r in ("gate", "up", "down")})
+        norms = lambda l: {"pre_mixer": norm(f"l{l}.n1"), "pre_ffn": norm(f"l{l}.n2")}
+        attn = AttentionSpec(H, nh, nkv, hd, hd ** -0.5, None, None, RotarySpec(hd, hd, 10000.0),
+                             {r: f"l1.attn.{r}" for r in "qkvo"})
+        layers = (BlockSpec("prenorm", DecaySpec(H, 0.75, "l0.mix.w"), ffn(0), norms(0)),
+                  BlockSpec("prenorm", attn, ffn(1), norms(1)))
+        return ModelPlan("ToyStateAndPagesLM", H, V, 256, EmbeddingSpec(V, H, 1.0, "emb"), layers,
+                         (LayerCall(0), LayerCall(1)), norm("final"), HeadSpec(V, H, None, "emb"))
+
+    with toy_architecture("ToyStateAndPagesLM", plan_of):
+        model = random_model({"architectures": ["ToyStateAndPagesLM"]}, "float32", seed=6, std=0.15,
+                             gain_std=0.1, rt=rt)
+        rng = np.random.default_rng(3)
+        prompts = [rng.integers(0, V, n).tolist() for n in (9, 14, 5, 11, 7, 13)]
+        sp = SamplingParams(max_tokens=12, temperature=0.0)
+        alone = []
+        for p in prompts:
+            eng = Engine(model, dtype="float32", block_size=4, num_blocks=64, max_batch_tokens=64,
+                         max_batch_seqs=2, prefill_chunk_size=5, max_seq_len=64)
+            alone.append(eng.generate([p], sp)[0])
+            eng.close()
+        # 9 pages of 4 tokens: one request needs up to 7, two that decode side by side up to 12
+        eng = Engine(model, dtype="float32", block_size=4, num_blocks=9, max_batch_tokens=64,
+                     max_batch_seqs=2, prefill_chunk_size=5, max_seq_len=64)
+        assert eng.runner.slot_bytes == H * 4 and len(eng.runner.manager.groups) == 1
+        admitted = []
+        clear = eng.runner.manager.on_admit
+        eng.runner.manager.on_admit = lambda r, s: (admitted.append((r, s)), clear(r, s))
+        together = eng.generate(prompts, sp)
+        assert together == alone
+        st = eng.stats()
+        assert st.preemptions > 0                                   # slots were taken again after giving up
+        assert len(admitted) >= len(prompts) + st.preemptions and {s for _, s in admitted} == {0, 1}
+        eng.runner.manager.check()
+        eng.close()

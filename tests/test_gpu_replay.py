@@ -66,20 +66,46 @@ def test_every_split_matches_the_plain_implementation(cases, name, dtype):
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_mixed_batches_with_pages_used_again(cases, name, dtype):
     folder, streams, refs = cases[(name, dtype)]
-    # room for the four longest live requests, each rounded up to 64: far less than all six
-    top4 = sorted((len(t) for t in streams.values()), reverse=True)[:4]
-    pool = sum(-(-n // 64) * 64 for n in top4)
-    assert pool < sum(-(-len(t) // PAGE[name]) * PAGE[name] for t in streams.values()) + 64
-    runner = make_runner(folder, dtype, page_size=PAGE[name], cache_tokens=pool, max_seqs=4,
+    page = PAGE[name]
+    pages_of = lambda n: -(-n // page)
+    # the pool holds the three longest requests and no more: strictly less than the six need
+    # together, so the later requests can only run on pages that earlier ones gave back
+    room = sum(sorted((pages_of(len(t)) for t in streams.values()), reverse=True)[:3])
+    assert room < sum(pages_of(len(t)) for t in streams.values()) - pages_of(max(len(t) for t in streams.values()))
+    runner = make_runner(folder, dtype, page_size=page, num_pages=room, max_seqs=4,
                          max_batch_tokens=256, max_model_len=256)
-    seen_pages = set()
+    m = runner.manager
+    assert [g.window is not None for g in m.groups] == [True, False]
+    assert all(p.num_pages == room for p in m.pools)
     for seed in (0, 1):
-        steps = mixed_steps(streams, seed=seed)
+        steps = mixed_steps(streams, seed=seed, room=room, page=page)
         assert max(len(e) for e, _ in steps) == 4
         assert any(any(n > 1 for _, n in e) and any(n == 1 for _, n in e) for e, _ in steps)
-        rows = run_steps(runner, streams, steps)
+        served = [dict() for _ in m.groups]           # per group: page -> requests it has served, in order
+        taken_from_the_living = [0 for _ in m.groups]
+
+        def observe(step_index):
+            live = set(m.live())
+            for g in range(len(m.groups)):
+                for r in live:
+                    for pg in m.table(r, g):
+                        if pg < 0:
+                            continue
+                        hist = served[g].setdefault(pg, [])
+                        if not hist or hist[-1] != r:
+                            # a page passes to r while the request that held it before still runs:
+                            # only a release by the window rule does that
+                            if hist and hist[-1] in live:
+                                taken_from_the_living[g] += 1
+                            hist.append(r)
+
+        rows = run_steps(runner, streams, steps, observe)
         check(rows, refs, dtype, f"mixed seed {seed}")
-        assert all(p.free_pages == p.num_pages for p in runner.manager.pools)
+        assert all(p.free_pages == p.num_pages for p in m.pools)
+        for g, info in enumerate(m.groups):
+            assert any(len(set(h)) >= 2 for h in served[g].values()), f"group {g}: no page was used again"
+        assert taken_from_the_living[0] > 0, "no page released by the window rule went to another live request"
+        assert taken_from_the_living[1] == 0       # the all-keys group gives pages back only at the end
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -189,3 +215,52 @@ def test_graph_replays_match_eager_steps(cases):
         assert np.array_equal(got, want), f"{r}: graph replay differs from the eager step"
         start = 20 + 7 * i
         assert_close(got, refs[r][start:start + len(got)], dtype, f"graph decode {r}")
+
+
+def test_a_decoded_tokens_bits_do_not_depend_on_the_batch_in_bfloat16(tmp_path):
+    """A request that decodes alone (bucket 1), beside seven others (bucket 8), through graphs
+    and eagerly, gets the same bits in bfloat16: the cut of the keys in the split attention is
+    fixed by the runner's limits, not by the batch.  The geometry is one where a rule that
+    looked at requests x KV heads x chunks (1 x 2 x 64 against 8 x 2 x 64) would change it."""
+    from zse_amd.engine.runner import StepEntry
+    from zse_amd.weights import write_random_model
+    cfg = dict(architectures=["Gemma2ForCausalLM"], model_type="gemma2", num_hidden_layers=2, hidden_size=64,
+               num_attention_heads=4, num_key_value_heads=2, head_dim=32, query_pre_attn_scalar=32,
+               intermediate_size=96, vocab_size=300, rope_theta=10000.0, sliding_window=16,
+               attn_logit_softcapping=30.0, final_logit_softcapping=20.0, rms_norm_eps=1e-6,
+               max_position_embeddings=4096)
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=5, std=0.08, gain_std=0.1, dtype="bfloat16",
+                                std_of={"embed_tokens": 0.02})
+    rng = np.random.default_rng(1)
+    main = rng.integers(0, 300, 150 + 6).tolist()
+    others = [rng.integers(0, 300, 40 + 13 * i + 6).tolist() for i in range(7)]
+
+    def run(use_graphs, crowd):
+        runner = make_runner(folder, "bfloat16", page_size=16, cache_tokens=2048, max_seqs=8,
+                             max_batch_tokens=256, max_model_len=4096, use_graphs=use_graphs)
+        mixer = runner.model.blocks[0].mixer
+        assert mixer.decode_chunk == 64               # 8 requests x 2 KV heads x 64 chunks
+        streams = {"main": main}
+        if crowd:
+            streams.update({f"o{i}": t for i, t in enumerate(others)})
+        for r, t in streams.items():
+            runner.step([StepEntry(r, t[:len(t) - 6], [])])
+        rows = []
+        for i in range(6):
+            z = runner.step([StepEntry(r, [t[len(t) - 6 + i]], [0]) for r, t in streams.items()])
+            rows.append(z[0])
+        if use_graphs:
+            assert any(isinstance(g, int) for g in runner.graphs.values())
+        return np.stack(rows)
+
+    alone_graph = run(True, False)
+    assert np.array_equal(alone_graph, run(False, False)), "graph and eager differ for a lone request"
+    assert np.array_equal(alone_graph, run(True, True)), "the crowd changed the request's bits (graphs)"
+    assert np.array_equal(alone_graph, run(False, True)), "the crowd changed the request's bits (eager)"
+    # a runner made for one request cuts the keys finer: near results, other bits allowed
+    small = make_runner(folder, "bfloat16", page_size=16, cache_tokens=512, max_seqs=1, max_batch_tokens=256,
+                        max_model_len=1024, use_graphs=False)
+    assert small.model.blocks[0].mixer.decode_chunk == 32
+    small.step([StepEntry("main", main[:150], [])])
+    z = small.step([StepEntry("main", [main[150]], [0])])
+    assert np.abs(z[0] - alone_graph[0]).max() < 0.02 * np.abs(alone_graph[0]).max()

@@ -136,11 +136,30 @@ def test_window_edge_is_i_minus_j_less_than_w():
     assert o[2, 0, 0] == 0.0                                          # causal: not before it exists
 
 
-def test_scale_and_cap_order():
-    # scale first, cap second: with a huge score the output saturates at cap
-    q = np.array([[[100.0]]]); k = np.array([[[100.0]]]); v = np.array([[[1.0]]])
-    s = P.softcap(np.array([100.0 * 100.0 * 0.5]), 50.0, F)
-    assert np.isclose(s, 50.0)
+def cap_order_vectors(hd=16):
+    """Two tokens, one head, chosen so that each wrong order of scale, cap and mask shows.
+    q1.k0 = 1e4, q1.k1 = 0, q0.k0 = -1e4; v0 = 1, v1 = 0; scale 0.01, cap 50.
+      right (scale, cap, mask): o1 = 1 / (1 + exp(-50 tanh 2)) = 1.000, o0 = 1 (sees key 0 only)
+      cap before scale:         o1 = 1 / (1 + exp(-0.5)) = 0.622
+      no cap:                   o1 = 1.000 too, but then o0's case below differs
+      mask before cap:          the hidden key 1 gets cap * tanh(-inf) = -50 beside key 0's
+                                -50 tanh 2 = -48.2:  o0 = 1 / (1 + exp(-1.8)) = 0.858"""
+    q = np.zeros((2, 1, hd)); k = np.zeros((2, 1, hd)); v = np.zeros((2, 1, hd))
+    q[0, 0, 0], q[1, 0, 0], k[0, 0, 0] = -100.0, 100.0, 100.0
+    v[0, 0, :] = 1.0
+    return q, k, v, 0.01, 50.0
+
+
+def test_scale_then_cap_then_mask_inside_attention():
+    q, k, v, scale, cap = cap_order_vectors()
+    o = P.attention(q, k, v, np.arange(2), scale, cap, None, F)
+    assert abs(o[1, 0, 0] - 1.0) < 1e-6          # 0.622 if the cap came before the scale
+    assert abs(o[0, 0, 0] - 1.0) < 1e-12         # 0.858 if the mask came before the cap
+    # and the cap is there at all: without it the same vectors give another o for a softer case
+    q2 = q / 10                                   # q1.k0 = 1e3 -> scaled 10, capped 9.87
+    o_cap = P.attention(q2, np.stack([k[0], k[0] * 0.9]), np.stack([v[0], v[1]]), np.arange(2), scale, 5.0, None, F)
+    # scores 10 and 9 scaled; capped at 5: 5 tanh 2 = 4.820 and 5 tanh 1.8 = 4.734: nearly a tie
+    assert abs(o_cap[1, 0, 0] - 1 / (1 + math.exp(5 * math.tanh(1.8) - 5 * math.tanh(2.0)))) < 1e-9
     assert P.visible(np.array([4]), np.arange(6), 3).tolist() == [[False, False, True, True, True, False]]
 
 

@@ -179,3 +179,63 @@ def test_no_starvation_under_random_load(seed):
     assert all(r.finished and r.finish_reason == FinishReason.LENGTH for r in rs)
     assert all(len(r.output_tokens) == r.params.max_tokens for r in rs)
     assert all(p.free_pages == p.num_pages for p in m.pools)
+
+
+def test_a_stop_token_found_after_preemption_ends_the_request_for_good():
+    # A run of steps leaves tokens on the device; the newest request is preempted while one of
+    # its tokens is still unknown, and that token turns out to be a stop token.  The request
+    # must leave the queue: it is never planned, computed or extended again.
+    s, m = make(pages=12, page=4, window=64, budget=64, chunk=16, seqs=4)
+    a, b = req("a", 7, 30), req("b", 7, 30, stop=[99])
+    s.add_request(a), s.add_request(b)
+    while not b.num_preemptions:
+        plan = s.schedule()
+        # ids still on the device: None stands for them, the output gets a placeholder
+        s.on_step_done(plan, {it.request.request_id: None for it in plan.items if it.sample})
+    assert b in s.waiting and b.state == RequestState.PREEMPTED
+    n = len(b.output_tokens)
+    assert n >= 2
+    b.output_tokens[n - 2] = 99                      # the ids arrive: the one before last ends b
+    assert s.finish_at(b, n - 1, FinishReason.STOP) is True
+    assert b.finished and b.finish_reason == FinishReason.STOP and len(b.output_tokens) == n - 1
+    assert b not in s.waiting and b not in s.running and s.finished["b"] is b
+    for _ in range(100):
+        if not s.has_work():
+            break
+        plan = s.schedule()
+        assert all(it.request is not b for it in plan.items)
+        s.on_step_done(plan, {it.request.request_id: 7 for it in plan.items if it.sample})
+        m.check()
+    assert not s.has_work() and a.finished and len(b.output_tokens) == n - 1
+    assert all(p.free_pages == p.num_pages for p in m.pools)
+    # a request that had already ended for another reason is not reported twice
+    assert s.finish_at(a, len(a.output_tokens), FinishReason.STOP) is False
+
+
+def test_every_admission_clears_the_state_slot():
+    # whoever makes a request live (first admission, or admission again after preemption),
+    # the owner of the slots' memory hears of it, with the slot the request got
+    s, m = make(pages=12, page=4, window=64, budget=64, chunk=16, seqs=2)
+    cleared = []
+    m.on_admit = lambda r, slot: cleared.append((r, slot))
+    rs = [req(i, 7, 20) for i in range(4)]
+    for r in rs:
+        s.add_request(r)
+    for _ in range(300):
+        if not s.has_work():
+            break
+        before = set(m.live())
+        run_step(s)
+        for r in set(m.live()) - before:
+            assert (r, m.slot(r)) in cleared
+    assert not s.has_work()
+    admissions = sum(1 + r.num_preemptions for r in rs)
+    assert sum(r.num_preemptions for r in rs) > 0 and len(cleared) >= admissions
+    assert {slot for _, slot in cleared} == {0, 1}          # two slots served four requests
+
+
+def test_penalty_counts_follow_the_continuous_batching_engine():
+    r = Request("p", [5, 5, 9], SamplingParams(max_tokens=8, repetition_penalty=1.3))
+    assert r.penalty_counts() == {5: 1, 9: 1}                # prompt tokens count once each
+    r.output_tokens += [9, 4, 4, 4]
+    assert r.penalty_counts() == {5: 1, 9: 2, 4: 3}          # produced tokens add up

@@ -41,6 +41,48 @@ def test_round_trip_and_header(tmp_path):
         assert "__metadata__" in json.loads(f.read(n))
 
 
+def test_reader_against_a_file_built_by_hand(tmp_path):
+    """The reader pinned without the writer: the bytes are put together here with struct.pack,
+    from the format's description as the reference reads it (format/convert.py:51-82: 8-byte
+    little-endian header length, JSON header, data_offsets relative to the end of the header,
+    __metadata__ skipped).  Offsets are out of order and the header is padded with spaces, as
+    real files are."""
+    import struct
+    f32 = [1.5, -2.0, 0.25, 3.0, 100.0, -0.125]                       # [2, 3] row-major
+    bf = [0x3F80, 0xC000, 0x3E80, 0x4049]                             # 1.0, -2.0, 0.25, 3.140625
+    f16 = [0x3C00, 0xB800]                                            # 1.0, -0.5
+    data_bf = struct.pack("<4H", *bf)
+    data_f32 = struct.pack("<6f", *f32)
+    data_f16 = struct.pack("<2H", *f16)
+    data = data_bf + data_f32 + data_f16                              # bf16 first in the file, listed last
+    header = {
+        "__metadata__": {"format": "pt"},
+        "w.f32": {"dtype": "F32", "shape": [2, 3], "data_offsets": [8, 32]},
+        "w.f16": {"dtype": "F16", "shape": [2], "data_offsets": [32, 36]},
+        "w.bf16": {"dtype": "BF16", "shape": [4, 1], "data_offsets": [0, 8]},
+    }
+    text = json.dumps(header).encode()
+    text += b" " * (-len(text) % 8)
+    p = tmp_path / "model.safetensors"
+    p.write_bytes(struct.pack("<Q", len(text)) + text + data)
+    h = st.read_header(str(p))
+    assert set(h) == {"w.f32", "w.f16", "w.bf16"}
+    assert h["w.f32"].shape == (2, 3) and h["w.bf16"].shape == (4, 1) and h["w.f16"].dtype == "F16"
+    assert np.array_equal(st.map_tensor(h["w.f32"]), np.array(f32, np.float32).reshape(2, 3))
+    assert st.map_tensor(h["w.bf16"]).reshape(-1).tolist() == bf
+    w = st.read_folder_f32(str(tmp_path))
+    assert w["w.bf16"].reshape(-1).tolist() == [1.0, -2.0, 0.25, 3.140625]
+    assert w["w.f16"].tolist() == [1.0, -0.5]
+    assert w["w.f32"][1].tolist() == [3.0, 100.0, -0.125]
+    # a header that points past the end of the file, or whose size disagrees with its shape
+    bad = dict(header)
+    bad["w.f32"] = {"dtype": "F32", "shape": [2, 3], "data_offsets": [8, 30]}
+    text2 = json.dumps(bad).encode()
+    (tmp_path / "model.safetensors").write_bytes(struct.pack("<Q", len(text2)) + text2 + data)
+    with pytest.raises(Exception):
+        st.map_tensor(st.read_header(str(p))["w.f32"])
+
+
 def test_no_safetensors_file_is_an_error(tmp_path):
     with pytest.raises(FileNotFoundError):
         st.index_folder(str(tmp_path))

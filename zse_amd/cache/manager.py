@@ -25,7 +25,7 @@ cache/cache_manager.py:269-283).
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Sequence
+from typing import Callable, Dict, List, Optional, Sequence
 
 import numpy as np
 
@@ -71,14 +71,21 @@ class CacheManager:
         self.max_model_len = int(max_model_len)
         self.max_blocks = -(-self.max_model_len // self.page_size)
         self._reqs: Dict[object, _Req] = {}
+        # called with (request, slot) whenever a request becomes live, whoever admits it (a
+        # scheduler, a step that meets a new request, a request computed again after giving
+        # everything up): the owner of the slots' memory clears the slot here
+        self.on_admit: Optional[Callable[[object, int], None]] = None
 
     # ---- requests
     def add(self, req) -> int:
-        """Admit a request: it gets a state slot (raises ``OutOfSlots``)."""
+        """Admit a request: it gets a state slot (raises ``OutOfSlots``), and the slot's
+        memory is cleared through ``on_admit``.  This is the only way a request becomes live."""
         if req in self._reqs:
             raise ValueError(f"request {req!r} is already live")
         slot = self.slots.acquire(req)
         self._reqs[req] = _Req(slot, 0, [[] for _ in self.groups], [0 for _ in self.groups])
+        if self.on_admit is not None:
+            self.on_admit(req, slot)
         return slot
 
     def has(self, req) -> bool:

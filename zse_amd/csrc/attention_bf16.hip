@@ -20,9 +20,10 @@
 // the same permutation.  V is therefore cached transposed, [page][kv head][hd][bs],
 // so that four consecutive keys of a channel are one 8-byte load.
 //
-// Decoded tokens use a split variant: the keys are cut into chunks of 64 aligned
-// to absolute positions, one wave per chunk writes (max, sum, O) and a second
-// kernel joins the chunks in order; the cut does not depend on the batch.  With
+// Decoded tokens use a split variant: the keys are cut into chunks of 64 (or 32, as
+// the caller says) aligned to absolute positions, one wave per chunk writes (max, sum, O)
+// and a second kernel joins the chunks in order; the cut is the caller's choice and never
+// follows from the batch, so a request's result is the same whoever shares its step.  With
 // at most 16 heads a KV head the chunks run on 16x16x32 MFMAs (attn_decode_kernel):
 // a single query token fills only g of a tile's columns, and the narrower tile
 // halves both the accumulator registers and the wasted work, so two waves fit a SIMD.
@@ -616,20 +617,49 @@ size_t zk_attention_bf16_workspace(int n_decode, int nh, int hd, int max_ctx) {
   return (size_t)n_decode * nh * nchunks * (hd + 2) * sizeof(float);
 }
 
+// Whether decoded tokens of these sizes run on the 16-wide tiles (partial results joined four
+// chunks at a time inside a block) or on the 32-wide ones (one partial result a chunk).
+static bool decode_on_narrow_tiles(int nh, int nkv, int hd) { return nh / nkv <= 16 && hd % 32 == 0; }
+
+// The longest context the split variant takes for decoded tokens (the joining kernel keeps one
+// weight per partial result in LDS).  ``decode_chunk`` as in zk_attention_bf16.
+long long zk_attention_bf16_max_context(int nh, int nkv, int hd, int decode_chunk) {
+  if (nkv <= 0 || nh % nkv) return 0;
+  const int chunk = decode_chunk == 32 ? 32 : ATT_CHUNK;
+  const long long span = decode_on_narrow_tiles(nh, nkv, hd) ? 4LL * chunk : ATT_CHUNK;
+  return span * ATT_MAX_CHUNKS;
+}
+
 // Requests [0, r_prefill) hold portions of more than one token (max_q_len the longest);
 // requests [r_prefill, R) hold one token each and use the split variant over max_ctx keys.
+// decode_chunk: keys a wave of the split variant takes on the 16-wide tiles, 32 or 64 (0: 64).
+// It fixes where the sums over keys are cut, and so the bits of the result: a caller that wants
+// a request's result not to depend on the rest of the batch passes the same value in every
+// step.  32 gives twice the waves, each with one load from memory in its chain instead of
+// two: better for few requests with short contexts, worse for many.
 int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const void* vcache_t,
                       const int* block_table, int max_blocks, const int* q_start, const int* ctx_len,
                       void* out, int R, int r_prefill, int max_q_len, int max_ctx, int nh, int nkv,
-                      int hd, int bs, float scale, float softcap, int window, void* workspace,
-                      size_t workspace_bytes, void* stream) {
+                      int hd, int bs, float scale, float softcap, int window, int decode_chunk,
+                      void* workspace, size_t workspace_bytes, void* stream) {
   ZK_REQUIRE(R >= 0 && r_prefill >= 0 && r_prefill <= R, "zk_attention_bf16: bad request counts");
   ZK_REQUIRE(zk_attention_bf16_supports(nh, nkv, hd, bs), "zk_attention_bf16: sizes not supported "
              "(head_dim 16/32/64/128/256, at most 32 heads a KV head, page size a power of two from 4)");
   ZK_REQUIRE(q_stride >= nh * hd && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0),
              "zk_attention_bf16: q rows must be 16-byte aligned");
   ZK_REQUIRE(max_blocks > 0 && nkv <= 65535 && R <= 65535, "zk_attention_bf16: grid too large");
+  ZK_REQUIRE(decode_chunk == 0 || decode_chunk == 32 || decode_chunk == 64,
+             "zk_attention_bf16: decode_chunk must be 32 or 64");
   if (R == 0) return 0;
+  // everything that can refuse is checked before the first launch
+  if (R - r_prefill > 0) {
+    ZK_REQUIRE(max_ctx > 0, "zk_attention_bf16: max_ctx must be positive");
+    ZK_REQUIRE(max_ctx <= zk_attention_bf16_max_context(nh, nkv, hd, decode_chunk),
+               "zk_attention_bf16: context too long for the split variant");
+    ZK_REQUIRE(zk_attention_bf16_workspace(R - r_prefill, nh, hd, max_ctx) <= workspace_bytes,
+               "zk_attention_bf16: workspace too small for the split partial results");
+  }
+  if (r_prefill > 0) ZK_REQUIRE(max_q_len > 0, "zk_attention_bf16: max_q_len must be positive");
   hipStream_t s = (hipStream_t)stream;
   AttnParams p;
   p.q = (const __bf16*)q; p.q_stride = q_stride;
@@ -646,7 +676,6 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
   p.c2 = softcap * log2e;
   const int g = nh / nkv;
   if (r_prefill > 0) {
-    ZK_REQUIRE(max_q_len > 0, "zk_attention_bf16: max_q_len must be positive");
     p.tpw = 32 / g; p.r_begin = 0; p.nchunks = 1; p.part_o = nullptr; p.part_ml = nullptr;
     const int groups = (max_q_len + p.tpw - 1) / p.tpw;
     // one block a group; two groups a block when that lets every block run at once (256 CUs,
@@ -659,10 +688,7 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
   }
   const int n_dec = R - r_prefill;
   if (n_dec > 0) {
-    ZK_REQUIRE(max_ctx > 0, "zk_attention_bf16: max_ctx must be positive");
     const int nchunks = (max_ctx + ATT_CHUNK - 1) / ATT_CHUNK;
-    ZK_REQUIRE(zk_attention_bf16_workspace(n_dec, nh, hd, max_ctx) <= workspace_bytes,
-               "zk_attention_bf16: workspace too small for the split partial results");
     p.tpw = 1; p.r_begin = r_prefill; p.nchunks = nchunks;
     p.part_o = (float*)workspace;
     p.part_ml = (float*)workspace + (size_t)n_dec * nh * nchunks * hd;
@@ -670,10 +696,8 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
     int rc = 0;
     int span = ATT_CHUNK;        // keys one partial result covers
     p.chunk = ATT_CHUNK;
-    if (g <= 16 && hd % 32 == 0) {
-      // Few requests and a short context give few waves (one request at 4096 keys: 256 for
-      // 256 CUs), each a chain of two loads from memory; half the keys a wave then, one load.
-      if ((long long)n_dec * nkv * nchunks <= 512) {
+    if (decode_on_narrow_tiles(nh, nkv, hd)) {
+      if (decode_chunk == 32) {
         p.chunk = ATT_CHUNK / 2;
         grid.x = (2 * nchunks + 3) / 4;
       }
@@ -693,7 +717,6 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
       rc = launch_attn<true, false>(p, grid, s);
     }
     if (rc) return rc;
-    ZK_REQUIRE(nchunks <= ATT_MAX_CHUNKS, "zk_attention_bf16: context too long for the split variant");
     dim3 cgrid(n_dec, nh);
     attn_combine_kernel<<<cgrid, 256, 0, s>>>(p.part_o, p.part_ml, q_start, ctx_len, (__bf16*)out, nh, hd,
                                               window, r_prefill, p.nchunks, span);

@@ -106,7 +106,7 @@ class Engine:
             if s.sample:
                 r = s.request
                 rows.append({"params": r.params, "u": uniform(r.seed, len(r.output_tokens)),
-                             "past": set(r.all_tokens) if r.params.repetition_penalty != 1.0 else ()})
+                             "past": r.penalty_counts() if r.params.repetition_penalty != 1.0 else ()})
                 who.append(r.request_id)
         ids = self.sampler.sample(logits, rows) if rows else []
         done = self.scheduler.on_step_done(plan, dict(zip(who, ids)))

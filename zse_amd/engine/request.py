@@ -57,6 +57,16 @@ class Request:
         """Tokens known but not yet in the cache."""
         return self.num_tokens - self.num_computed
 
+    def penalty_counts(self) -> dict:
+        """Token id -> count for the repetition penalty, as the reference's continuous-batching
+        engine keeps it: every token of the prompt counts once however often it occurs
+        (zstreamer/engine.py:441), every produced token adds one (zstreamer/request.py:164).
+        The sampler scales the penalty by these counts (orchestrator/sampler.py:64-74)."""
+        counts = {int(t): 1 for t in self.prompt_tokens}
+        for t in self.output_tokens:
+            counts[int(t)] = counts.get(int(t), 0) + 1
+        return counts
+
     @property
     def finished(self) -> bool:
         return self.state == RequestState.FINISHED

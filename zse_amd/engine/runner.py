@@ -179,10 +179,22 @@ class StepRunner:
         self.slot_bytes = slot_bytes
         self.manager = CacheManager(groups, self.page_size, self.max_seqs, self.max_model_len, slot_bytes)
         self.state = rt.zeros((self.max_seqs, max(slot_bytes // 4, 1)), F32) if slot_bytes else None
+        self.manager.on_admit = self._clear_slot
 
         # ---- step buffers
         self.arena = Arena(rt)
-        self.workspace = rt.zeros((self._workspace_words(),), F32)
+        # one workspace for every part's kernels (a launch at a time uses it): each part says
+        # what it needs at this runner's limits, and refuses limits it cannot serve, here
+        need = 0
+        for part in model.parts():
+            need = max(need, int(part.prepare(self.k, self.dtype, self.max_seqs, self.max_model_len,
+                                              self.page_size)))
+        try:
+            self.workspace = rt.zeros((max(need // 4 + 1, 64),), F32)
+        except Exception as e:
+            raise RuntimeError(f"the kernels' workspace for {self.max_seqs} requests of up to "
+                               f"{self.max_model_len} tokens needs {need} bytes and cannot be "
+                               f"allocated: {e}") from None
         self.gemm_workspace = None
         if self.dtype == BF16 and self.k.has("zk_gemm_bf16_workspace"):
             self.gemm_workspace = rt.zeros((self.k.zk_gemm_bf16_workspace() // 4,), F32)
@@ -195,14 +207,14 @@ class StepRunner:
         rt.record(self.meta_copied)
         self.logits: Optional[Tensor] = None
         self.graphs: Dict[int, object] = {}      # bucket -> "warm" | graph handle
+        # a captured step replays the same launches with the same arguments: every part must
+        # take what changes from step to step (tokens, positions, tables, slots) from device
+        # memory alone.  The built-in parts do; a part says so with ``graph_safe = True``.
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in model.parts())
         self.graph_logits: Optional[Tensor] = None
         self.steps_run = 0
 
     # ------------------------------------------------------------------ sizes
-    def _workspace_words(self) -> int:
-        # partial results of split attention: sized by the bf16 kernels' own need
-        return 1 << 20 if self.dtype == F32 else (32 << 20)
-
     def _meta_words(self, T: int, R: int, G: int) -> int:
         return 4 * T + (R + 1) + 2 * R + G * (T + R * self.max_blocks) + 64
 
@@ -210,11 +222,15 @@ class StepRunner:
         return sum(c.k.nbytes + c.v.nbytes for c in self.caches if c.k is not None)
 
     # ------------------------------------------------------------------ requests
-    def add(self, req) -> int:
-        slot = self.manager.add(req)
+    def _clear_slot(self, req, slot: int) -> None:
+        """A request became live (the manager calls this, whoever admitted it): its state slot
+        starts from zero.  The clearing kernel runs on the runner's stream, after the steps
+        that the slot's last owner took part in and before the first step of the new one."""
         if self.state is not None:
             self.rt.zero_(self.state.rows(slot, slot + 1))
-        return slot
+
+    def add(self, req) -> int:
+        return self.manager.add(req)
 
     def finish(self, req) -> None:
         self.manager.release(req)
@@ -315,7 +331,7 @@ class StepRunner:
     def _graph_bucket(self, entries) -> int:
         """The padded batch size under which a decode-only step replays a captured graph
         (0: run eagerly).  Every entry brings one token and wants its logits."""
-        if not self.use_graphs or self.state is not None:
+        if not self.use_graphs or not self.graph_safe:
             return 0
         if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
             return 0

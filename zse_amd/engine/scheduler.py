@@ -206,16 +206,24 @@ class Scheduler:
     def finish_at(self, req: Request, length: int, reason: FinishReason) -> bool:
         """A token that was still unknown when the request was stepped on turned out to end
         it: cut its output to ``length`` tokens and finish it now.  Returns True if the request
-        was still running."""
+        was still running or waiting to run again (it is then reported as done by the caller),
+        False if it had already finished for another reason."""
         del req.output_tokens[length:]
-        was_running = req in self.running
-        if was_running:
-            self.manager.release(req.request_id)
+        was_live = False
+        if req in self.running:
             self.running.remove(req)
+            was_live = True
+        elif req in self.waiting:
+            # preempted after the step that drew the token, before the token was known: it
+            # must not be admitted and computed again
+            self.waiting.remove(req)
+            was_live = True
+        if was_live:
+            self.manager.release(req.request_id)      # a request in the queue holds nothing: a no-op
             self.finished[req.request_id] = req
         req.state = RequestState.FINISHED
         req.finish_reason = reason
-        return was_running
+        return was_live
 
     def stats(self) -> dict:
         return {"waiting": len(self.waiting), "running": len(self.running),

@@ -21,6 +21,8 @@ from .ops import linear, tuned_gemm
 
 
 class PagedAttention(Part):
+    graph_safe = True      # its launches take what changes from step to step from device memory alone
+
     def __init__(self, spec):
         s = self.spec = spec
         if s.num_heads % s.num_kv_heads:
@@ -30,6 +32,7 @@ class PagedAttention(Part):
         self.position = build_part("position", s.position)
         self.shared_kv = "k" not in s.names        # reads another call's cache, writes none
         self.w_qkv = self.w_o = None
+        self.decode_chunk = 64                     # keys a wave of the split decode attention takes
 
     def children(self):
         return [self.position]
@@ -61,6 +64,25 @@ class PagedAttention(Part):
         s = self.spec
         return bool(dtype == BF16 and kernels.has("zk_attention_bf16") and
                     kernels.zk_attention_bf16_supports(s.num_heads, s.num_kv_heads, s.head_dim, page_size))
+
+    def prepare(self, kernels, dtype, max_seqs, max_model_len, page_size) -> int:
+        """Workspace of the split attention of decoded tokens at the runner's limits, and the
+        number of keys a wave of it takes.  That number fixes where the sums over keys are cut:
+        it follows from the limits alone, never from a step's batch, so a request's result does
+        not depend on who shares its step."""
+        s = self.spec
+        if not self.wants_v_transposed(kernels, dtype, page_size):
+            return 0
+        chunks = -(-int(max_model_len) // 64)
+        self.decode_chunk = 32 if int(max_seqs) * s.num_kv_heads * chunks <= 512 else 64
+        longest = int(kernels.zk_attention_bf16_max_context(s.num_heads, s.num_kv_heads, s.head_dim,
+                                                            self.decode_chunk))
+        if max_model_len > longest:
+            raise ValueError(f"attention with {s.num_heads} heads, {s.num_kv_heads} KV heads of "
+                             f"{s.head_dim}: the longest context its decode kernel takes is {longest} "
+                             f"tokens, the runner asks for {max_model_len}")
+        return int(kernels.zk_attention_bf16_workspace(int(max_seqs), s.num_heads, s.head_dim,
+                                                       int(max_model_len)))
 
     def forward(self, ctx, x: Tensor, cache) -> Tensor:
         s, k = self.spec, ctx.k
@@ -97,7 +119,7 @@ class PagedAttention(Part):
             k.zk_attention_bf16(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
                                 ctx.q_start, ctx.ctx_len, o.ptr, ctx.R, ctx.n_multi, ctx.max_q_len,
                                 ctx.max_ctx, nh, nkv, hd, g.page_size, s.scale, cap, win,
-                                ctx.workspace.ptr, ctx.workspace.nbytes, ctx.stream)
+                                self.decode_chunk, ctx.workspace.ptr, ctx.workspace.nbytes, ctx.stream)
         else:
             k.zk_attention_plain(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table,
                                  g.max_blocks, ctx.req_of_token, ctx.positions, o.ptr, T, nh, nkv,

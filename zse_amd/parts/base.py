@@ -53,6 +53,11 @@ class StateNeed:
 
 class Part:
     spec = None
+    # True: every launch of the part reads what differs between steps (tokens, positions, block
+    # tables, slots) from device memory, so a captured decode step may be replayed.  A part that
+    # looks at the step's host-side description (``ctx.entries``) leaves this False, and the
+    # runner then runs every step eagerly.
+    graph_safe = False
 
     def tensor_reqs(self) -> List[TensorReq]:
         return []
@@ -62,6 +67,13 @@ class Part:
 
     def children(self) -> List["Part"]:
         return []
+
+    def prepare(self, kernels, dtype: str, max_seqs: int, max_model_len: int, page_size: int) -> int:
+        """Called once by the step runner, with its limits, before the first step.  A part
+        fixes here whatever must not change from step to step, refuses limits its kernels
+        cannot serve (with the numbers, at construction and not in the middle of a run) and
+        returns the bytes of the runner's shared workspace its kernels need for one launch."""
+        return 0
 
 
 _REGISTRIES: Dict[str, Dict[str, Callable]] = {

@@ -17,6 +17,8 @@ ARRANGEMENTS = {"sandwich": ("pre_mixer", "post_mixer", "pre_ffn", "post_ffn"),
 
 
 class Block(Part):
+    graph_safe = True      # its launches take what changes from step to step from device memory alone
+
     def __init__(self, spec):
         if spec.arrangement not in ARRANGEMENTS:
             raise ValueError(f"arrangement must be one of {sorted(ARRANGEMENTS)}, got {spec.arrangement!r}")

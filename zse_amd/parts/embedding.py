@@ -19,6 +19,8 @@ from .ops import linear, tuned_gemm
 
 
 class Embedding(Part):
+    graph_safe = True      # its launches take what changes from step to step from device memory alone
+
     def __init__(self, spec):
         self.spec = spec
         self.table = None
@@ -49,6 +51,8 @@ class Embedding(Part):
 
 
 class LMHead(Part):
+    graph_safe = True      # its launches take what changes from step to step from device memory alone
+
     def __init__(self, spec):
         self.spec = spec
         self.weight = None

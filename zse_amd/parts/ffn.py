@@ -17,6 +17,8 @@ ACTIVATION_CODES = {"gelu_tanh": 0, "silu": 1}
 
 
 class GatedMLP(Part):
+    graph_safe = True      # its launches take what changes from step to step from device memory alone
+
     def __init__(self, spec):
         if spec.activation not in ACTIVATION_CODES:
             raise ValueError(f"activation must be one of {sorted(ACTIVATION_CODES)}, got {spec.activation!r}")

@@ -13,6 +13,8 @@ from .base import ROLE_GAIN, Part, TensorReq, register_part
 
 
 class RMSNorm(Part):
+    graph_safe = True      # its launches take what changes from step to step from device memory alone
+
     def __init__(self, spec):
         self.spec = spec
         self.weight: Optional[Tensor] = None

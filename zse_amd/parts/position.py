@@ -14,6 +14,8 @@ from .base import Part, register_part
 
 
 class Rotary(Part):
+    graph_safe = True      # its launches take what changes from step to step from device memory alone
+
     def __init__(self, spec):
         if spec.rotary_dim % 2 or not (0 < spec.rotary_dim <= spec.head_dim):
             raise ValueError(f"rotary_dim must be even and in (0, head_dim], got {spec.rotary_dim}")
@@ -36,6 +38,8 @@ class Rotary(Part):
 
 
 class NoPosition(Part):
+    graph_safe = True      # its launches take what changes from step to step from device memory alone
+
     def __init__(self, spec):
         self.spec = spec
 

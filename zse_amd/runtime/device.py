@@ -165,7 +165,7 @@ BF16_KERNEL_SIGNATURES = {
     "zk_strip_layout": [_VP, _VP, _I, _I, _VP],
     "zk_qkv_rope_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "zk_attention_bf16": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
-                          _F, _F, _I, _VP, _SZ, _VP],
+                          _F, _F, _I, _I, _VP, _SZ, _VP],
 }
 
 
@@ -199,6 +199,9 @@ class KernelLibrary:
             self._dll.zk_attention_bf16_workspace.restype = C.c_size_t
             self._dll.zk_attention_bf16_workspace.argtypes = [_I, _I, _I, _I]
             self.zk_attention_bf16_workspace = self._dll.zk_attention_bf16_workspace
+            self._dll.zk_attention_bf16_max_context.restype = C.c_longlong
+            self._dll.zk_attention_bf16_max_context.argtypes = [_I, _I, _I, _I]
+            self.zk_attention_bf16_max_context = self._dll.zk_attention_bf16_max_context
             self._dll.zk_qkv_rope_bf16_supports.restype = C.c_int
             self._dll.zk_qkv_rope_bf16_supports.argtypes = [_I, _I, _I, _I]
             self.zk_qkv_rope_bf16_supports = self._dll.zk_qkv_rope_bf16_supports
