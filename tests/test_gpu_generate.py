@@ -234,7 +234,7 @@ def test_a_crowd_of_mixed_requests_each_gets_what_it_gets_alone(tiny_folders, se
         eng.close()
         return out, st
 
-    crowd, st = run(range(24), 5, 22)
+    crowd, st = run(range(24), 5, 14)        # 14 pages of 8: the longest request alone needs 9
     assert st.preemptions > 0, "the pool was meant to be too small for five long requests"
     roomy = Engine(folder, dtype="float32", block_size=8, num_blocks=64, max_batch_tokens=48, max_batch_seqs=1,
                    prefill_chunk_size=16, max_seq_len=128, decode_run=1)

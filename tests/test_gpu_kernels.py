@@ -800,3 +800,44 @@ def test_cut_offs_on_awkward_rows(rt):
         got = sampler.sample(rt.upload(z), rows)
         want = [sample_host(z[i], r["params"], r["u"]) for i, r in enumerate(rows)]
         assert got == want, [(i, g, w) for i, (g, w) in enumerate(zip(got, want)) if g != w]
+
+
+# ------------------------------------------------------------------ random weights
+@pytest.mark.parametrize("n", [1, 2, 7, 4096, 1_000_003])
+def test_device_random_weights_equal_the_host_function_bit_for_bit(rt, n):
+    from zse_amd.weights.normal import normal
+    from zse_amd.weights.safetensors import f32_to_bf16_bits
+    for seed, stream, mean, std in [(0, 1234567, 0.0, 0.02), (2 ** 40 + 3, 2 ** 32 - 1, 0.5, 1.0)]:
+        want = normal(n, seed, stream, mean, std)
+        for dtype in ("float32", "bfloat16"):
+            k = rt.kernels(dtype)
+            out32 = rt.zeros((n,), "float32")
+            k.zk_fill_normal(out32.ptr, 0, n, seed, stream, mean, std, rt.stream)
+            got = rt.download(out32)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (
+                f"{dtype} library, float output: first difference at {np.argmax(got != want)}")
+        outb = rt.zeros((n,), "bfloat16")
+        rt.kernels("bfloat16").zk_fill_normal(outb.ptr, 1, n, seed, stream, mean, std, rt.stream)
+        assert np.array_equal(rt.download(outb), f32_to_bf16_bits(want))
+
+
+def test_a_model_made_on_the_device_equals_the_folder_written_on_the_host(rt, tmp_path):
+    """Same configuration, seed and deviations: ``random_model`` (weights drawn by the device in
+    place) and ``write_random_model`` + ``load_model`` (drawn on the host, written, read, copied)
+    are the same model: the same logits, bit for bit, in both types."""
+    from conftest import TINY
+    from zse_amd.engine.loading import load_model, random_model
+    from zse_amd.engine.runner import StepEntry, StepRunner
+    from zse_amd.weights import write_random_model
+    cfg = TINY["B"][0]
+    toks = np.random.default_rng(0).integers(0, cfg["vocab_size"], 19).tolist()
+    for dtype in ("float32", "bfloat16"):
+        folder = write_random_model(str(tmp_path / dtype), cfg, seed=21, std=0.07, gain_std=0.15, dtype=dtype,
+                                    std_of={"embed_tokens": 0.02})
+        rows = []
+        for model in (load_model(folder, dtype, rt),
+                      random_model(cfg, dtype, seed=21, std=0.07, gain_std=0.15, rt=rt, std_of={"embed_tokens": 0.02})):
+            runner = StepRunner(model, rt, dtype, page_size=8, cache_tokens=64, max_seqs=2, max_batch_tokens=64,
+                                max_model_len=64, use_graphs=False)
+            rows.append(runner.step([StepEntry("a", toks, range(len(toks)))]))
+        assert np.abs(rows[0]).max() > 0.1 and np.array_equal(rows[0], rows[1]), dtype

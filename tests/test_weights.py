@@ -155,3 +155,24 @@ def test_unsupported_dtype_is_reported(tmp_path):
     with pytest.raises(WeightError) as e:
         check_folder(d, reqs_of(TINY_A))
     assert e.value.wrong_dtype == [("model.norm.weight", "I32")]
+
+
+def test_the_random_weights_function():
+    """Values are a function of (seed, stream, element index) alone: any slice can be made
+    by itself, other seeds and streams give other values, and the values are standard normal
+    (the device makes the same bits; tests/test_gpu_kernels.py compares them)."""
+    from zse_amd.weights.normal import normal, normal_tensor, stream_of
+    x = normal(400_001, 9, 77)
+    assert x.dtype == np.float32 and x.shape == (400_001,)
+    assert np.array_equal(normal(1001, 9, 77, first=12_345), x[12_345:13_346])       # odd start, odd count
+    assert np.array_equal(normal(2, 9, 77, first=400_000 - 1), x[-2:])
+    assert not np.array_equal(normal(100, 10, 77), x[:100]) and not np.array_equal(normal(100, 9, 78), x[:100])
+    assert abs(float(x.mean())) < 0.01 and abs(float(x.std()) - 1) < 0.01
+    assert abs(float((x.astype(np.float64) ** 4).mean()) - 3) < 0.1 and 4 < np.abs(x).max() < 6
+    # the two values of a pair are not correlated, nor are neighbours
+    assert abs(np.corrcoef(x[0:-1:2], x[1::2])[0, 1]) < 0.01 and abs(np.corrcoef(x[1:-1], x[2:])[0, 1]) < 0.01
+    y = normal(50_000, 9, 77, mean=1.5, std=0.02)
+    assert abs(float(y.mean()) - 1.5) < 1e-3 and abs(float(y.std()) - 0.02) < 1e-3
+    assert stream_of("layers.0.mlp.up_proj.weight") != stream_of("layers.1.mlp.up_proj.weight")
+    t = normal_tensor((7, 5), 1, "a.b")
+    assert t.shape == (7, 5) and np.array_equal(t.reshape(-1), normal(35, 1, stream_of("a.b")))

@@ -455,21 +455,83 @@ __device__ __forceinline__ uint64_t mix64(uint64_t z) {
   return z ^ (z >> 31);
 }
 
-// Normal(mean, std) values as a pure function of (seed, stream, element index).
+// Normal(mean, std) values as a pure function of (seed, stream, element index), by Box-Muller.
+// The host can make the very same values (zse_amd/weights/normal.py): logarithm, sine and cosine
+// are written out here as short sums of single correctly rounded float operations (no library
+// call, no fused multiply-add: contraction is off in these functions), so that NumPy, doing the
+// same operations in the same order, gets the same bits.
+//
+//   r = mix64(mix64(seed ^ stream * C) + pair);  k = (r >> 40) + 1 in [1, 2^24];  j = (r >> 8) & (2^24 - 1)
+//   u1 = k / 2^24,  angle = 2 pi j / 2^24
+//   element 2 pair = mean + std * sqrt(-2 ln u1) * cos(angle), element 2 pair + 1 the same with sin
+
+// ln(k / 2^24) for an integer k in [1, 2^24]: k = m * 2^e with m in [1/sqrt2, sqrt2),
+// ln m = 2 atanh(s) = 2 s (1 + s^2/3 + s^4/5 + s^6/7 + s^8/9), s = (m - 1) / (m + 1).
+__device__ __forceinline__ float exact_log_u24(uint32_t k) {
+#pragma clang fp contract(off)
+  int e = 31 - __clz((int)k);
+  float m = (float)k * __int_as_float((127 - e) << 23);       // k / 2^e, exact: k has at most 24 bits
+  if (m > 1.41421354f) {
+    m = m * 0.5f;
+    e += 1;
+  }
+  const float s = (m - 1.0f) / (m + 1.0f);
+  const float s2 = s * s;
+  float p = 0.111111112f;
+  p = p * s2 + 0.142857149f;
+  p = p * s2 + 0.2f;
+  p = p * s2 + 0.333333343f;
+  p = p * s2 + 1.0f;
+  const float lm = (2.0f * s) * p;
+  return (float)(e - 24) * 0.693147182f + lm;
+}
+
+// sin and cos of 2 pi j / 2^24 for an integer j in [0, 2^24): the quarter turn and the fold to
+// [0, pi/4] are integer work, the rest two short polynomials in x = r * (pi / 2^23), r <= 2^21.
+__device__ __forceinline__ void exact_sincos_u24(uint32_t j, float& sn, float& cs) {
+#pragma clang fp contract(off)
+  const uint32_t q = j >> 22;
+  uint32_t r = j & 0x3FFFFFu;
+  const bool fold = r > 0x200000u;
+  if (fold) r = 0x400000u - r;
+  const float x = (float)r * 3.74507039e-07f;                 // pi / 2 / 2^22
+  const float x2 = x * x;
+  float ps = 2.75573188e-06f;                                 // 1/9!
+  ps = ps * x2 + -1.98412701e-04f;                            // -1/7!
+  ps = ps * x2 + 8.33333377e-03f;                             // 1/5!
+  ps = ps * x2 + -1.66666672e-01f;                            // -1/3!
+  const float s0 = x + (x * x2) * ps;
+  float pc = -2.75573188e-07f;                                // -1/10!
+  pc = pc * x2 + 2.48015876e-05f;                             // 1/8!
+  pc = pc * x2 + -1.38888892e-03f;                            // -1/6!
+  pc = pc * x2 + 4.16666679e-02f;                             // 1/4!
+  pc = pc * x2 + -0.5f;
+  const float c0 = 1.0f + x2 * pc;
+  const float s1 = fold ? c0 : s0, c1 = fold ? s0 : c0;       // sin(pi/2 - x) = cos x
+  switch (q) {
+    case 0: sn = s1; cs = c1; break;
+    case 1: sn = c1; cs = -s1; break;
+    case 2: sn = -s1; cs = -c1; break;
+    default: sn = -c1; cs = s1; break;
+  }
+}
+
 template <typename D>
 __global__ void fill_normal_kernel(D* __restrict__ dst, size_t n, uint64_t seed, uint64_t stream,
                                    float mean, float std) {
+#pragma clang fp contract(off)
   size_t pair = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   size_t i = pair * 2;
   if (i >= n) return;
   uint64_t r = mix64(mix64(seed ^ (stream * 0xD1342543DE82EF95ull)) + pair);
-  const float u1 = ((float)(uint32_t)(r >> 40) + 1.0f) * (1.0f / 16777216.0f);  // (0, 1]
-  const float u2 = (float)(uint32_t)((r >> 8) & 0xFFFFFF) * (1.0f / 16777216.0f);
-  const float rad = sqrtf(-2.0f * logf(u1));
+  const uint32_t k = (uint32_t)(r >> 40) + 1u;
+  const uint32_t j = (uint32_t)((r >> 8) & 0xFFFFFFu);
+  const float rad = sqrtf(-2.0f * exact_log_u24(k));     // correctly rounded, as NumPy's
   float sn, cs;
-  sincosf(6.283185307179586f * u2, &sn, &cs);
-  dst[i] = from_f32<D>(mean + std * rad * cs);
-  if (i + 1 < n) dst[i + 1] = from_f32<D>(mean + std * rad * sn);
+  exact_sincos_u24(j, sn, cs);
+  const float a = std * (rad * cs), b = std * (rad * sn);
+  dst[i] = from_f32<D>(mean + a);
+  if (i + 1 < n) dst[i + 1] = from_f32<D>(mean + b);
 }
 
 __global__ void zero_kernel(uint32_t* __restrict__ p, size_t n_words) {

@@ -29,15 +29,16 @@ def load_model(model_dir: str, dtype: str, rt: Optional[Runtime] = None, tuned: 
 
 
 def random_model(config: dict, dtype: str, seed: int = 0, std: float = 0.02, gain_std: float = 0.1,
-                 rt: Optional[Runtime] = None, tuned: bool = True) -> Model:
-    """A model with seeded random weights made on the device (no folder is written)."""
+                 rt: Optional[Runtime] = None, tuned: bool = True, std_of=None) -> Model:
+    """A model with seeded random weights made on the device (no folder is written): the same
+    weights that ``write_random_model`` writes for the same configuration, seed and deviations."""
     rt = rt or Runtime.get()
     dtype = canonical_dtype(dtype)
     arch = resolve_architecture(config)
     typed = arch.config_from_dict(config)
     model = Model(arch.plan(typed))
     model.config = typed
-    src = RandomWeights(rt, dtype, model.tensor_reqs(), seed, std, gain_std, tuned=tuned)
+    src = RandomWeights(rt, dtype, model.tensor_reqs(), seed, std, gain_std, tuned=tuned, std_of=std_of)
     model.load(src, rt, dtype)
     model.tuned = bool(tuned)
     rt.sync()

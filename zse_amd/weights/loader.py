@@ -187,20 +187,31 @@ class RandomWeights(_Source):
     N(0, gain_std); each value is a function of (seed, tensor name, index)."""
 
     def __init__(self, rt, dtype: str, reqs: Iterable[TensorReq], seed: int, std: float = 0.02,
-                 gain_std: float = 0.1, tuned: bool = True):
+                 gain_std: float = 0.1, tuned: bool = True, std_of=None):
         super().__init__(rt, dtype, tuned)
         self.reqs = merge_reqs(reqs)
         self.seed, self.std, self.gain_std = int(seed), float(std), float(gain_std)
+        self.std_of = dict(std_of or {})
 
     def _shape(self, name):
         return self.reqs[_strip(name)].shape
 
     def _fill(self, name: str, dst: Tensor, dst_kind: int):
-        import zlib
+        from .normal import stream_of
+        from .random_init import deviation_of
         r = self.reqs[_strip(name)]
-        std = r.init_std if r.init_std is not None else (self.gain_std if r.role == ROLE_GAIN else self.std)
-        self.k.zk_fill_normal(dst.ptr, dst_kind, dst.numel, self.seed,
-                              zlib.crc32(_strip(name).encode()), 0.0, std, self.rt.stream)
+        std = deviation_of(r, self.std, self.gain_std, self.std_of)
+        if dst_kind == 0 and self.dtype == BF16:
+            # a vector kept as float32 in a bfloat16 model holds what a bfloat16 checkpoint
+            # would: values rounded to bfloat16 (so the model equals the folder written on the host)
+            tmp = self.rt.empty((dst.numel,), BF16)
+            self.k.zk_fill_normal(tmp.ptr, 1, dst.numel, self.seed, stream_of(_strip(name)), 0.0, std,
+                                  self.rt.stream)
+            self.k.zk_convert(tmp.ptr, SRC_TAGS["BF16"], dst.ptr, 0, dst.numel, self.rt.stream)
+            self.rt.sync()
+            return
+        self.k.zk_fill_normal(dst.ptr, dst_kind, dst.numel, self.seed, stream_of(_strip(name)), 0.0, std,
+                              self.rt.stream)
 
     def close(self):
         pass

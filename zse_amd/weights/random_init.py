@@ -1,16 +1,18 @@
 """Random-weights mode: a model folder (config.json, model.safetensors) from a
 configuration and a seed.
 
-Values are drawn on the host with a seeded generator, one stream per tensor
-name, so a tensor's values do not depend on the other tensors: matrices
-N(0, std), gains N(0, gain_std).  The reference has no such mode for models
-(random weights appear only in its adapter tests, orchestrator/lora_manager.py:157).
+Values are a pure function of (seed, tensor name, element index): matrices
+N(0, std), gains N(0, gain_std), so a tensor's values do not depend on the other
+tensors.  The function is the one the device uses when it makes a model's weights
+in place (``zk_fill_normal``; ``zse_amd.weights.normal`` computes the same bits on
+the host): a folder written here and a model made on the device from the same
+configuration and seed hold the same weights.  The reference has no such mode for
+models (random weights appear only in its adapter tests, orchestrator/lora_manager.py:157).
 """
 from __future__ import annotations
 
 import json
 import os
-import zlib
 from typing import Optional
 
 import numpy as np
@@ -19,18 +21,23 @@ from ..config.base import ARCHITECTURES, resolve_architecture
 from ..parts.base import ROLE_GAIN
 from . import safetensors as st
 from .loader import merge_reqs
+from .normal import normal_tensor
+
+
+def deviation_of(req, std: float, gain_std: float, std_of=None) -> float:
+    """The deviation a tensor is drawn with: its own if the part names one, else the mode's
+    for its role; ``std_of`` maps a piece of a tensor name to a deviation and wins."""
+    s = req.init_std if req.init_std is not None else (gain_std if req.role == ROLE_GAIN else std)
+    for part, v in (std_of or {}).items():
+        if part in req.name:
+            s = v
+    return float(s)
 
 
 def random_tensors(reqs, seed: int, std: float, gain_std: float, std_of=None):
-    out = {}
-    for key, r in merge_reqs(reqs).items():
-        rng = np.random.Generator(np.random.Philox(key=[int(seed), zlib.crc32(key.encode())]))
-        s = r.init_std if r.init_std is not None else (gain_std if r.role == ROLE_GAIN else std)
-        for part, v in (std_of or {}).items():
-            if part in r.name:
-                s = v
-        out[r.name] = (rng.standard_normal(r.shape, dtype=np.float32) * np.float32(s))
-    return out
+    """{name: float32 array} for every tensor the parts ask for (one draw per name)."""
+    return {r.name: normal_tensor(r.shape, seed, key, 0.0, deviation_of(r, std, gain_std, std_of))
+            for key, r in merge_reqs(reqs).items()}
 
 
 def write_random_model(out_dir: str, config: dict, seed: int = 0, std: float = 0.02,
