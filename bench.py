@@ -1,21 +1,36 @@
 #!/usr/bin/env python3
-"""Decode and prefill throughput of Gemma 2 2B layer shapes on one MI355X.
+"""Decode and prefill throughput of Gemma 2 layer shapes on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+    python bench.py --workload 9b|27b
 
-A step is one decode step of the whole batch: every live request brings one token, the
-model runs from the cache, the next token is picked greedily on the device.  Weights are
-seeded random values, token ids are synthetic.  One JSON line comes out; its ``value`` is
-decoded tokens a second at the default batch, ``points`` holds batch 1 and 64, ``prefill``
-one 2,048-token prompt in one step, ``roofline`` the decode step's bytes over its time.
+The default run times Gemma 2 2B shapes.  A step is one decode step of the whole batch: every
+live request brings one token, the model runs from the cache, the next token is picked greedily
+on the device.  Weights are seeded random values, token ids are synthetic.  One JSON line comes
+out; its ``value`` is decoded tokens a second at the default batch, ``points`` holds batch 1
+and 64, ``prefill`` one 2,048-token prompt in one step, ``roofline`` the decode step's bytes
+over its time.  Fractions are given against the published peaks (``frac``) and against what
+two probe kernels reach on this very GPU (``frac_probed``).
+
+Before anything is timed the model is checked (``checked``): a two-layer slice of the very
+model that is timed (same seed, so the same tensors) runs whole prompts, portions and single
+tokens in 32-bit and in bfloat16 against the plain implementation under ``tests/plain`` on the
+same weights made on the host, and the full model's decode steps through captured graphs must
+pick the same tokens as eager steps.  A failed check ends the run with an error.
+
+``--workload`` runs one of the two larger workloads through ``Engine.generate`` instead, end to
+end: 9b = 32 requests with prompts of 128 to 4,096 tokens, 256 greedy tokens each, portions of
+512; 27b = 8 prompts of 8,192 tokens, 128 tokens each at temperature 1.0, seed 3.
 """
 import argparse
 import json
+import os
 import sys
 import time
 
 import numpy as np
 
+ROOT = os.path.dirname(os.path.abspath(__file__))
 PEAK_HBM = 8.0e12          # bytes/s, MI355X
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
@@ -27,7 +42,7 @@ GEMMA2_2B = dict(
     max_position_embeddings=8192)
 
 
-# further sizes of the same architecture, for looking beyond the default (--model)
+# further sizes of the same architecture, for looking beyond the default (--model, --workload)
 GEMMA2_9B = dict(GEMMA2_2B, num_hidden_layers=42, hidden_size=3584, num_attention_heads=16, num_key_value_heads=8,
                  head_dim=256, query_pre_attn_scalar=256, intermediate_size=14336)
 GEMMA2_27B = dict(GEMMA2_2B, num_hidden_layers=46, hidden_size=4608, num_attention_heads=32, num_key_value_heads=16,
@@ -52,7 +67,8 @@ def cache_bytes(cfg, ctx, item=2):
     return total
 
 
-def prefill_flops(cfg, T):
+def prefill_flops(cfg, T, start=0):
+    """Flops of a step that brings tokens [start, start + T) of one request and wants one row."""
     H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
     nh, nkv, hd, L, W = (cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"],
                          cfg["num_hidden_layers"], cfg["sliding_window"])
@@ -60,10 +76,204 @@ def prefill_flops(cfg, T):
     gemm = 2.0 * T * per_layer * L
     attn = 0.0
     for l in range(L):
-        w = W if (l % 2 == 0 and W) else T
-        keys = sum(min(i + 1, w) for i in range(T))
+        w = W if (l % 2 == 0 and W) else start + T
+        keys = sum(min(i + 1, w) for i in range(start, start + T))
         attn += 4.0 * nh * hd * keys
     return gemm + attn + 2.0 * V * H
+
+
+def log(msg):
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+# ------------------------------------------------------------------ what this GPU reaches
+def probe_peaks(rt):
+    """(bytes/s a kernel streams from memory, bf16 flop/s of the matrix cores alone), each the
+    best of a few launches of a probe kernel."""
+    import ctypes
+    k = rt.kernels("bfloat16")
+    sink = rt.zeros((64,), "float32")
+    nbytes = 4 << 30
+    buf = rt.zeros((nbytes // 4,), "float32")
+    a, b = rt.event(), rt.event()
+    best_bw = 0.0
+    for _ in range(6):
+        rt.record(a)
+        k.zk_probe_read(buf.ptr, nbytes, sink.ptr, rt.stream)
+        rt.record(b)
+        best_bw = max(best_bw, nbytes / (rt.elapsed_ms(a, b) * 1e-3))
+    flops = ctypes.c_double(0.0)
+    best_fl = 0.0
+    for _ in range(4):
+        rt.record(a)
+        k.zk_probe_mfma_bf16(4000, sink.ptr, ctypes.byref(flops), rt.stream)
+        rt.record(b)
+        best_fl = max(best_fl, flops.value / (rt.elapsed_ms(a, b) * 1e-3))
+    return best_bw, best_fl
+
+
+# ------------------------------------------------------------------ the check before timing
+def bf16_round(a):
+    from zse_amd.weights.safetensors import bf16_bits_to_f32, f32_to_bf16_bits
+    return bf16_bits_to_f32(f32_to_bf16_bits(np.ascontiguousarray(a, np.float32)))
+
+
+def check_slice(cfg, rt, seed, std, gain_std):
+    """Layers 0 and 1, embedding, final norm and head of the model that is timed (the same
+    tensors: a tensor's values follow from seed, name and index) against the plain
+    implementation, in 32-bit and in bfloat16, cut three ways.  The host makes the same weights
+    with the host side of the random-weights function.  The plain head is restricted to the
+    first 8,192 rows of the embedding (token ids are drawn below that), whose logits are
+    compared; the product over the whole vocabulary has a test of its own."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from plain import gemma2_plain as P
+    from zse_amd.engine.loading import random_model
+    from zse_amd.engine.model import Model
+    from zse_amd.engine.runner import StepEntry, StepRunner
+    from zse_amd.config.base import resolve_architecture
+    from zse_amd.weights.random_init import random_tensors
+
+    small = dict(cfg, num_hidden_layers=2)
+    Vc = min(8192, cfg["vocab_size"])
+    host_cfg = dict(small, vocab_size=Vc)
+    arch = resolve_architecture(host_cfg)
+    w32 = random_tensors(Model(arch.plan(arch.config_from_dict(host_cfg))).tensor_reqs(), seed, std, gain_std)
+    rng = np.random.default_rng(11)
+    streams = {"a": rng.integers(0, Vc, 40).tolist(), "b": rng.integers(0, Vc, 37).tolist(),
+               "c": rng.integers(0, Vc, 21).tolist()}
+    # a whole; b in portions of 9, 2 and 13, then token by token beside c's portions and tokens
+    steps = [[("a", 40)], [("b", 9)], [("b", 2), ("c", 5)], [("b", 13), ("c", 1)]]
+    steps += [[("b", 1), ("c", 3 if i == 0 else 1)] for i in range(13)]
+    out = {}
+    for dtype in ("float32", "bfloat16"):
+        w = w32 if dtype == "float32" else {n: bf16_round(t) for n, t in w32.items()}
+        model = random_model(small, dtype, seed=seed, std=std, gain_std=gain_std, rt=rt)
+        runner = StepRunner(model, rt, dtype, page_size=16, cache_tokens=512, max_seqs=4, max_batch_tokens=256,
+                            max_model_len=256, use_graphs=False)
+        fed = {r: 0 for r in streams}
+        rows = {r: [] for r in streams}
+        for st in steps:
+            es = [StepEntry(r, streams[r][fed[r]:fed[r] + n], range(n)) for r, n in st if fed[r] < len(streams[r])]
+            z = runner.step(es)
+            at = 0
+            for e in es:
+                n = len(e.tokens)
+                rows[e.req].append(z[at:at + n, :Vc])
+                at += n
+                fed[e.req] += n
+        assert all(fed[r] == len(t) for r, t in streams.items()), fed
+        worst = 0.0
+        for r, toks in streams.items():
+            want = P.forward(host_cfg, w, toks, np.float64)
+            got = np.concatenate(rows[r]).astype(np.float64)
+            err = np.abs(got - want).max() / max(1.0, np.abs(want).max())
+            worst = max(worst, float(err))
+        out[dtype] = worst
+        del runner, model
+    return out
+
+
+def check_graphs(model, rt, vocab):
+    """The model that is timed: tokens picked through captured decode steps equal those of eager steps."""
+    from zse_amd.engine.runner import StepEntry, StepRunner
+    rng = np.random.default_rng(5)
+    prompts = [rng.integers(0, vocab, 24 + 3 * i).tolist() for i in range(8)]
+    picked = []
+    for graphs in (False, True):
+        runner = StepRunner(model, rt, "bfloat16", page_size=16, cache_tokens=1024, max_seqs=8, max_batch_tokens=512,
+                            max_model_len=4096, use_graphs=graphs)
+        z = runner.step([StepEntry(i, p, [len(p) - 1]) for i, p in enumerate(prompts)])
+        ids = [z.argmax(axis=1).tolist()]
+        for _ in range(6):
+            z = runner.step([StepEntry(i, [t], [0]) for i, t in enumerate(ids[-1])])
+            ids.append(z.argmax(axis=1).tolist())
+        if graphs and not any(isinstance(g, int) for g in runner.graphs.values()):
+            raise SystemExit("bench.py: no decode step was captured into a graph")
+        picked.append(ids)
+        del runner
+    return picked[0] == picked[1]
+
+
+# ------------------------------------------------------------------ workloads through the engine
+def run_workload(name, a):
+    from zse_amd.engine.engine import Engine
+    from zse_amd.engine.loading import random_model
+    from zse_amd.runtime.device import Runtime
+    from zse_amd.sampling import SamplingParams
+    cfg = dict(MODELS[name])
+    full_layers = cfg["num_hidden_layers"]
+    if a.layers:
+        cfg["num_hidden_layers"] = a.layers
+    if name == "27b":
+        # the workload's prompts fill Gemma 2's 8,192 positions by themselves: room for the new tokens
+        cfg["max_position_embeddings"] = 8192 + 128
+    rt = Runtime.get()
+    t0 = time.time()
+    model = random_model(cfg, "bfloat16", seed=0, std=0.02, gain_std=0.1, rt=rt)
+    log(f"{name}: model ready in {time.time() - t0:.1f} s, {model.weight_bytes / 1e9:.2f} GB of weights")
+    rng = np.random.default_rng(0)
+    V, page = cfg["vocab_size"], 16
+    if name == "9b":
+        lengths = rng.integers(128, 4097, 32).tolist()
+        params = SamplingParams(max_tokens=256, temperature=0.0)
+        what = "32 requests, prompts uniform in [128, 4096], 256 greedy tokens each, portions of 512"
+    else:
+        lengths = [8192] * 8
+        params = SamplingParams(max_tokens=128, temperature=1.0, seed=3)
+        what = "8 prompts of 8192 tokens, 128 tokens each at temperature 1.0 (seed 3), portions of 512"
+    prompts = [rng.integers(0, V, n).tolist() for n in lengths]
+    n_new = params.max_tokens
+    max_len = max(lengths) + n_new
+    blocks = sum(-(-(n + n_new) // page) for n in lengths) + 8
+    eng = Engine(model, dtype="bfloat16", block_size=page, num_blocks=blocks, max_batch_tokens=4096,
+                 max_batch_seqs=len(prompts), prefill_chunk_size=512, max_seq_len=max_len)
+    # a small run first: code objects load, the arena and the first graphs are made
+    eng.generate([p[:70] for p in prompts[:2]], SamplingParams(max_tokens=6, temperature=0.0))
+    m = eng.runner.manager
+    stats0 = eng.stats()
+    stats0.by_kind.clear(), stats0.ttft_ms.clear(), stats0.tpot_ms.clear()
+    stats0.peak_pages = [0] * len(m.pools)
+    steps0, gen0, sec0 = stats0.steps, stats0.generated_tokens, stats0.seconds
+    rt.sync()
+    t1 = time.perf_counter()
+    out = eng.generate(prompts, params)
+    rt.sync()
+    dt = time.perf_counter() - t1
+    st = eng.stats()
+    assert all(len(o) == n_new for o in out)
+    gen = st.generated_tokens - gen0
+    prompt_tokens = sum(lengths)
+    needs = model.cache_needs()
+    item = 2
+    groups = []
+    for g, pool, peak in zip(m.groups, m.pools, st.peak_pages):
+        per_page = sum(2 * needs[c].num_kv_heads * needs[c].head_dim for c in g.calls) * item * page
+        groups.append({"window": g.window, "layers": len(g.calls), "pages": pool.num_pages, "peak_pages": peak,
+                       "peak_gb": round(peak * per_page / 1e9, 2), "pool_gb": round(pool.num_pages * per_page / 1e9, 2)})
+    # what the cache would hold at the end without the window rule: every layer keeps every key
+    per_token_all = sum(2 * n.num_kv_heads * n.head_dim for n in needs if n is not None) * item
+    no_release_gb = sum(-(-(n + n_new) // page) * page for n in lengths) * per_token_all / 1e9
+    kinds = {k: {"steps": int(v[0]), "tokens": int(v[1]), "seconds": round(v[2], 3),
+                 "ms_per_step": round(1e3 * v[2] / max(v[0], 1), 3)} for k, v in st.by_kind.items()}
+    res = {
+        "metric": f"end-to-end generated tok/s, Gemma 2 {name.upper()} bf16 workload", "value": round(gen / dt, 1),
+        "unit": "tok/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+        "workload": what, "seconds": round(dt, 3), "generated_tokens": gen, "prompt_tokens": prompt_tokens,
+        "all_tokens_per_s": round((gen + prompt_tokens) / dt, 1), "steps": st.steps - steps0,
+        "preemptions": st.preemptions,
+        "config": {"model": f"gemma2-{name}-shapes-random", "layers": cfg["num_hidden_layers"], "layers_full": full_layers,
+                   "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+                   "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+                   "intermediate": cfg["intermediate_size"], "vocab": V, "sliding_window": cfg["sliding_window"],
+                   "requests": len(prompts), "max_tokens": n_new, "page_size": page, "prefill_chunk_size": 512,
+                   "max_batch_tokens": 4096, "max_positions": cfg["max_position_embeddings"],
+                   "weights_gb": round(model.weight_bytes / 1e9, 2)},
+        "by_kind": kinds, "cache_groups": groups, "cache_without_window_release_gb": round(no_release_gb, 2),
+        "ttft_ms_mean": round(float(np.mean(st.ttft_ms)), 1), "ttft_ms_max": round(float(np.max(st.ttft_ms)), 1),
+        "tpot_ms_mean": round(float(np.mean(st.tpot_ms)), 3),
+    }
+    eng.close()
+    print(json.dumps(res), flush=True)
 
 
 def main():
@@ -77,13 +287,18 @@ def main():
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated")
     ap.add_argument("--model", choices=sorted(MODELS), default="2b", help="layer sizes: Gemma 2 2B (the default), 9B or 27B")
+    ap.add_argument("--workload", choices=["9b", "27b"], default=None,
+                    help="run one of the larger workloads through Engine.generate instead")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--no-check", action="store_true", help="profiling aid: skip the check before timing")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="profiling aid: run one of the two workloads (the JSON line then lacks the other)")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not measured")
         sys.exit(2)
+    if a.workload:
+        return run_workload(a.workload, a)
 
     from zse_amd.engine.loading import random_model
     from zse_amd.engine.runner import StepEntry, StepRunner
@@ -95,8 +310,26 @@ def main():
     if a.layers:
         cfg["num_hidden_layers"] = a.layers
     rt = Runtime.get()
+    SEED, STD, GAIN_STD = 0, 0.02, 0.1
+
     t0 = time.time()
-    model = random_model(cfg, "bfloat16", seed=0, std=0.02, gain_std=0.1, rt=rt)
+    model = random_model(cfg, "bfloat16", seed=SEED, std=STD, gain_std=GAIN_STD, rt=rt)
+    V = cfg["vocab_size"]
+    check = None
+    if not a.no_check and not a.only:
+        errs = check_slice(cfg, rt, SEED, STD, GAIN_STD)
+        same_ids = check_graphs(model, rt, V)
+        # 32-bit: summation order only (2e-5 of the largest logit seen at these widths);
+        # bfloat16: inputs of every product rounded to 8 bits (under 1 % seen)
+        ok = errs["float32"] < 1e-4 and errs["bfloat16"] < 0.02 and same_ids
+        check = {"fp32_max_rel_err": float(f"{errs['float32']:.3g}"), "bf16_max_rel_err": float(f"{errs['bfloat16']:.3g}"),
+                 "graph_ids_equal_eager": bool(same_ids), "slice_layers": 2, "cuts": "whole, portions, token by token, mixed"}
+        log(f"check: {check} ({time.time() - t0:.1f} s)")
+        if not ok:
+            raise SystemExit(f"bench.py: the engine does not agree with the plain implementation: {check}")
+    peak_bw, peak_fl = probe_peaks(rt)
+    log(f"probes: {peak_bw / 1e9:.0f} GB/s streamed, {peak_fl / 1e12:.0f} TFLOP/s bf16 on the matrix cores")
+
     points = sorted({int(x) for x in a.points.split(",") if x} | {a.batch})
     max_b = max(points)
     page = 16
@@ -107,11 +340,9 @@ def main():
                         use_graphs=not a.no_graphs)
     sampler = DeviceSampler(rt, runner.k, max_b)
     greedy = SamplingParams(temperature=0.0)
-    V = cfg["vocab_size"]
     rng = np.random.default_rng(0)
-    print(f"[bench] model ready in {time.time() - t0:.1f} s: {cfg['num_hidden_layers']} layers, "
-          f"{model.weight_bytes / 1e9:.2f} GB of weights, cache {runner.cache_bytes() / 1e9:.2f} GB",
-          file=sys.stderr, flush=True)
+    log(f"model ready in {time.time() - t0:.1f} s: {cfg['num_hidden_layers']} layers, "
+        f"{model.weight_bytes / 1e9:.2f} GB of weights, cache {runner.cache_bytes() / 1e9:.2f} GB")
 
     # ---- prefill: one prompt of 2,048 tokens in one step
     T = a.prefill_tokens
@@ -129,8 +360,8 @@ def main():
         pre_s = float(np.median(times[1:]))
         pf = prefill_flops(cfg, T)
         prefill = {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
-                   "frac": round(pf / pre_s / PEAK_FLOPS["bf16"], 4)}
-        print(f"[bench] prefill {T} tokens: {pre_s * 1e3:.2f} ms", file=sys.stderr, flush=True)
+                   "frac": round(pf / pre_s / PEAK_FLOPS["bf16"], 4), "frac_probed": round(pf / pre_s / peak_fl, 4)}
+        log(f"prefill {T} tokens: {pre_s * 1e3:.2f} ms")
     if a.only == "prefill":
         print(json.dumps({"prefill": prefill}), flush=True)
         return
@@ -184,8 +415,8 @@ def main():
         k = a.steps if B == a.batch else max(16, a.steps // 2)
         w = a.warmup if B == a.batch else max(4, a.warmup // 2)
         results[B] = decode(B, k, w)
-        print(f"[bench] decode batch {B}: {results[B][0]:.1f} tok/s, {results[B][1] * 1e3:.3f} ms/step, "
-              f"{results[B][2] / results[B][1] / 1e9:.0f} GB/s", file=sys.stderr, flush=True)
+        log(f"decode batch {B}: {results[B][0]:.1f} tok/s, {results[B][1] * 1e3:.3f} ms/step, "
+            f"{results[B][2] / results[B][1] / 1e9:.0f} GB/s")
 
     tok_s, step_s, byts = results[a.batch]
     out = {
@@ -202,8 +433,12 @@ def main():
                    "graphs": int(runner.use_graphs)},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(byts / step_s / 1e9, 1), "peak": PEAK_HBM / 1e9,
-                     "unit": "GB/s", "frac": round(byts / step_s / PEAK_HBM, 4)},
+                     "unit": "GB/s", "frac": round(byts / step_s / PEAK_HBM, 4),
+                     "frac_probed": round(byts / step_s / peak_bw, 4)},
         "points": {f"decode_b{B}": round(results[B][0], 1) for B in points if B != a.batch},
+        "points_roofline_frac": {f"decode_b{B}": round(results[B][2] / results[B][1] / PEAK_HBM, 4) for B in points},
+        "probed": {"hbm_gbs": round(peak_bw / 1e9, 1), "mfma_bf16_tflops": round(peak_fl / 1e12, 1)},
+        "checked": check is not None, "check": check,
     }
     print(json.dumps(out), flush=True)
 

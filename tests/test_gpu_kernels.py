@@ -802,6 +802,43 @@ def test_cut_offs_on_awkward_rows(rt):
         assert got == want, [(i, g, w) for i, (g, w) in enumerate(zip(got, want)) if g != w]
 
 
+# ------------------------------------------------------------------ the LM head at full size
+def test_lm_head_product_at_full_vocabulary(rt):
+    """N = 256,000 rows of K = 2,304 in strip layout (1.18 GB, 16,000 strips), soft cap in the
+    epilogue, float logits: every row count the engine uses (skinny 1 and 8, mid 40, tile 200)
+    against the plain product on 3,000 sampled columns, the first and last strips among them."""
+    from zse_amd.weights.normal import normal
+    from zse_amd.weights.safetensors import f32_to_bf16_bits
+    k = rt.kernels("bfloat16")
+    N, K, cap, seed, stream = 256000, 2304, 30.0, 5, 99
+    W = rt.empty((N, K), "bfloat16")
+    k.zk_fill_normal(W.ptr, 1, N * K, seed, stream, 0.0, 0.05, rt.stream)
+    Ws = rt.empty((N, K), "bfloat16")
+    k.zk_strip_layout(W.ptr, Ws.ptr, N, K, rt.stream)
+    rt.sync()
+    rng = np.random.default_rng(3)
+    cols = np.unique(np.concatenate([np.arange(0, 40), np.arange(N - 40, N), rng.integers(0, N, 2920),
+                                     [65535, 65536, 131071, 131072]]))
+    w_cols = np.stack([normal(K, seed, stream, 0.0, 0.05, first=int(c) * K) for c in cols])      # the same rows, made on the host
+    Wc = rt.upload(f32_to_bf16_bits(w_cols), "bfloat16")
+    ws = gemm_workspace(rt)
+    for M in (1, 8, 40, 200):
+        a = bf16(rng.normal(size=(M, K)))
+        A = up(rt, a, "bfloat16")
+        want = rt.empty((M, len(cols)), "float32")
+        k.zk_gemm_plain(A.ptr, K, Wc.ptr, want.ptr, len(cols), 1, M, len(cols), K, rt.stream)
+        want = rt.download(want).astype(np.float64)
+        want = cap * np.tanh(want / cap)
+        got = rt.zeros((M, N), "float32")
+        k.zk_gemm_bf16(A.ptr, K, Ws.ptr, got.ptr, N, 1, M, N, K, 1, cap, 1, ws.ptr, ws.nbytes, None, rt.stream)
+        got = rt.download(got)
+        assert np.abs(want).max() > 5 and np.all(np.abs(got) < cap)
+        err = np.abs(got[:, cols] - want)
+        assert err.max() < 1e-4 * math.sqrt(K), f"M={M}: {err.max()} at column {cols[err.max(axis=0).argmax()]}"
+        # no column outside the sample is left unwritten or wildly off: each has the spread of a logit
+        assert np.all(got.std(axis=0) > 0) if M >= 8 else np.count_nonzero(got) > N * 0.99
+
+
 # ------------------------------------------------------------------ random weights
 @pytest.mark.parametrize("n", [1, 2, 7, 4096, 1_000_003])
 def test_device_random_weights_equal_the_host_function_bit_for_bit(rt, n):

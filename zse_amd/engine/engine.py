@@ -30,10 +30,29 @@ class EngineStats:
     generated_tokens: int = 0
     preemptions: int = 0
     seconds: float = 0.0
+    # per kind of step ("prefill": prompt portions only, "decode": single tokens only,
+    # "mixed": both): [steps, tokens, seconds on the host's clock]
+    by_kind: Dict[str, List[float]] = field(default_factory=dict)
+    peak_pages: List[int] = field(default_factory=list)        # most pages in use at once, per cache group
+    # per finished request, with the reference's meanings (zstreamer/request.py:206-228)
+    ttft_ms: List[float] = field(default_factory=list)
+    tpot_ms: List[float] = field(default_factory=list)
 
     @property
     def tokens_per_second(self) -> float:
         return self.generated_tokens / self.seconds if self.seconds > 0 else 0.0
+
+    def note_step(self, kind: str, steps: int, tokens: int, seconds: float) -> None:
+        e = self.by_kind.setdefault(kind, [0, 0, 0.0])
+        e[0] += steps
+        e[1] += tokens
+        e[2] += seconds
+
+    def note_finished(self, reqs) -> None:
+        for r in reqs:
+            if r.finish_reason is not None and r.finish_reason.value != "error":
+                self.ttft_ms.append(r.ttft_ms)
+                self.tpot_ms.append(r.tpot_ms)
 
 
 class Engine:
@@ -46,17 +65,10 @@ class Engine:
         self.dtype = canonical_dtype(dtype)
         self.model = load_model(model, self.dtype, self.rt, tuned=tuned) if isinstance(model, str) else model
         max_len = min(max_seq_len or self.model.plan.max_position, self.model.plan.max_position)
-        if num_blocks is None:
-            # enough for every request slot at a moderate length, bounded by memory left
-            per_token = sum(2 * n.num_kv_heads * n.head_dim for n in self.model.cache_needs()
-                            if n is not None and hasattr(n, "num_kv_heads"))
-            per_token *= 2 if self.dtype == "bfloat16" else 4
-            free = self.rt.info().free_memory
-            want_tokens = max_batch_seqs * max_len
-            fit_tokens = int(free * 0.6) // max(per_token, 1)
-            num_blocks = max(1, min(want_tokens, fit_tokens) // block_size)
+        pages = self._pages_per_group(num_blocks, block_size, max_batch_seqs, max_len,
+                                      min(prefill_chunk_size, max_batch_tokens))
         self.runner = StepRunner(self.model, self.rt, self.dtype, page_size=block_size,
-                                 num_pages=num_blocks, max_seqs=max_batch_seqs,
+                                 num_pages=pages, max_seqs=max_batch_seqs,
                                  max_batch_tokens=max_batch_tokens, max_model_len=max_len,
                                  use_graphs=use_graphs)
         self.scheduler = Scheduler(SchedulerConfig(max_batch_tokens, prefill_chunk_size, max_batch_seqs),
@@ -70,6 +82,30 @@ class Engine:
         # device; a stop token found afterwards cuts the request's output back to it.
         self.decode_run = max(1, min(int(decode_run), DeviceSampler.RING))     # results on their way at a time
         self._next_plan: Optional[StepPlan] = None
+
+    def _pages_per_group(self, num_blocks: Optional[int], block_size: int, max_seqs: int, max_len: int,
+                         step_tokens: int) -> List[int]:
+        """Pages for each cache group, in the runner's order of groups.  A group that keeps
+        every key gets ``num_blocks`` pages (not given: enough for every request slot at the
+        longest context, as far as 60 % of the free memory goes).  A windowed group gets what
+        its requests can hold at most: the window, the page that is leaving it and the tokens
+        of one step, for every request slot; never more than the all-keys number."""
+        from ..cache.manager import group_needs
+        needs = self.model.cache_needs()
+        groups = group_needs(needs)
+        item = 2 if self.dtype == "bfloat16" else 4
+        def bytes_per_page(g):
+            return sum(2 * needs[c].num_kv_heads * needs[c].head_dim for c in g.calls) * item * block_size
+        def windowed_pages(g):
+            per_request = -(-(g.window + step_tokens) // block_size) + 2
+            return max_seqs * min(per_request, -(-max_len // block_size))
+        if num_blocks is None:
+            budget = int(self.rt.info().free_memory * 0.6)
+            budget -= sum(windowed_pages(g) * bytes_per_page(g) for g in groups if g.window is not None)
+            full = sum(bytes_per_page(g) for g in groups if g.window is None)
+            want = max_seqs * -(-max_len // block_size)
+            num_blocks = max(1, min(want, budget // full if full else want))
+        return [min(num_blocks, windowed_pages(g)) if g.window is not None else num_blocks for g in groups]
 
     # ---- requests
     def add_request(self, prompt_tokens: Sequence[int], params: Optional[SamplingParams] = None,
@@ -89,10 +125,27 @@ class Engine:
         return req
 
     def step(self) -> List[Request]:
-        """Schedule, run and sample one step; returns the requests that finished in it."""
+        """Schedule, run and sample one step (or a run of decode steps); returns the requests
+        that finished in it."""
+        t0 = time.monotonic()
         plan, self._next_plan = self._next_plan or self.scheduler.schedule(), None
         if not plan:
             return list(plan.failed)
+        pools = self.runner.manager.pools
+        if len(self._stats.peak_pages) != len(pools):
+            self._stats.peak_pages = [0] * len(pools)
+        self._stats.peak_pages = [max(a, p.used_pages) for a, p in zip(self._stats.peak_pages, pools)]
+        multi = any(s.count > 1 for s in plan.items)
+        single = any(s.count == 1 and s.request.state == RequestState.DECODING for s in plan.items)
+        kind = "mixed" if multi and single else ("prefill" if multi or not single else "decode")
+        steps0, tokens = self._stats.steps, plan.num_tokens
+        done = self._step(plan)
+        n = self._stats.steps - steps0
+        self._stats.note_step(kind, n, tokens * max(n, 1), time.monotonic() - t0)
+        self._stats.note_finished(done)
+        return done
+
+    def _step(self, plan: StepPlan) -> List[Request]:
         run = self._run_length(plan)
         if run >= 2:
             return self._decode_run(plan, run)

@@ -10,6 +10,7 @@ the cache.
 from __future__ import annotations
 
 import enum
+import time
 from dataclasses import dataclass, field
 from typing import List, Optional
 
@@ -43,6 +44,10 @@ class Request:
     error: Optional[str] = None
     arrival: int = 0
     num_preemptions: int = 0
+    # clock readings (time.monotonic) for the timing figures below
+    arrival_time: float = 0.0
+    first_token_time: Optional[float] = None
+    finish_time: Optional[float] = None
 
     @property
     def all_tokens(self) -> List[int]:
@@ -66,6 +71,31 @@ class Request:
         for t in self.output_tokens:
             counts[int(t)] = counts.get(int(t), 0) + 1
         return counts
+
+    # ---- timing, with the reference's names and meanings (zstreamer/request.py:206-228)
+    @property
+    def total_time_ms(self) -> float:
+        return ((self.finish_time or time.monotonic()) - self.arrival_time) * 1000.0
+
+    @property
+    def ttft_ms(self) -> float:
+        """Time to the first token; the whole time for a request that never produced one."""
+        if self.first_token_time is None:
+            return self.total_time_ms
+        return (self.first_token_time - self.arrival_time) * 1000.0
+
+    @property
+    def tpot_ms(self) -> float:
+        """Mean time per output token after the first."""
+        if self.first_token_time is None:
+            return self.total_time_ms
+        end = self.finish_time or time.monotonic()
+        return (end - self.first_token_time) * 1000.0 / max(len(self.output_tokens), 1)
+
+    @property
+    def tokens_per_sec(self) -> float:
+        total = self.total_time_ms
+        return max(len(self.output_tokens), 1) / (total / 1000.0) if total > 0 else 0.0
 
     @property
     def finished(self) -> bool:

@@ -150,8 +150,14 @@ class StepRunner:
         if num_pages is None:
             tokens = cache_tokens if cache_tokens is not None else self.max_model_len
             num_pages = -(-int(tokens) // self.page_size)
-        for g in groups:
-            g.num_pages = int(num_pages)
+        # one number for every group, or one per group in the groups' order (windowed groups
+        # first, by window; the all-keys group last): a windowed group never holds more than
+        # its window and a step's tokens per request, so its pool can be much the smaller
+        per_group = list(num_pages) if isinstance(num_pages, (list, tuple)) else [num_pages] * len(groups)
+        if len(per_group) != len(groups):
+            raise ValueError(f"{len(per_group)} page counts for {len(groups)} cache groups")
+        for g, n in zip(groups, per_group):
+            g.num_pages = int(n)
         slot_bytes = 0
         self.caches: List[CallCache] = []
         gid_of = {}
@@ -163,13 +169,14 @@ class StepRunner:
             cc = CallCache(need=need)
             if isinstance(need, PagedKV):
                 cc.group = gid_of[i]
-                shape = (num_pages, need.num_kv_heads, self.page_size, need.head_dim)
+                pages = groups[cc.group].num_pages
+                shape = (pages, need.num_kv_heads, self.page_size, need.head_dim)
                 cc.k = rt.zeros(shape, self.dtype)
                 mixer = model.blocks[model.plan.order[i].layer].mixer
                 cc.v_transposed = bool(self.tuned and getattr(mixer, "wants_v_transposed", None) and
                                        mixer.wants_v_transposed(self.k, self.dtype, self.page_size))
                 if cc.v_transposed:
-                    shape = (num_pages, need.num_kv_heads, need.head_dim, self.page_size)
+                    shape = (pages, need.num_kv_heads, need.head_dim, self.page_size)
                 cc.v = rt.zeros(shape, self.dtype)
             elif isinstance(need, StateNeed):
                 cc.state_offset = slot_bytes

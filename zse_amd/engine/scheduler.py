@@ -23,6 +23,7 @@ not fit, it ends with an error.  Admission never preempts.
 """
 from __future__ import annotations
 
+import time
 from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, List, Optional, Tuple
@@ -85,6 +86,7 @@ class Scheduler:
             raise ValueError(f"request {req.request_id!r}: prompt of {len(req.prompt_tokens)} tokens "
                              f"exceeds the longest context, {self.manager.max_model_len}")
         req.arrival = self._arrivals
+        req.arrival_time = time.monotonic()
         self._arrivals += 1
         req.state = RequestState.WAITING
         self.waiting.append(req)
@@ -115,6 +117,7 @@ class Scheduler:
             self.running.remove(req)
         req.state = RequestState.FINISHED
         req.finish_reason = FinishReason.ERROR
+        req.finish_time = time.monotonic()
         req.error = why
         self.finished[req.request_id] = req
         plan.failed.append(req)
@@ -186,6 +189,8 @@ class Scheduler:
             known = sampled[req.request_id] is not None
             tok = int(sampled[req.request_id]) if known else UNKNOWN_TOKEN     # still on the device: set later
             req.output_tokens.append(tok)
+            if req.first_token_time is None:
+                req.first_token_time = time.monotonic()
             req.state = RequestState.DECODING
             reason = None
             if known and req.params.stop_tokens and tok in req.params.stop_tokens:
@@ -197,6 +202,7 @@ class Scheduler:
             if reason is not None:
                 req.state = RequestState.FINISHED
                 req.finish_reason = reason
+                req.finish_time = time.monotonic()
                 self.manager.release(req.request_id)
                 self.running.remove(req)
                 self.finished[req.request_id] = req
@@ -223,6 +229,7 @@ class Scheduler:
             self.finished[req.request_id] = req
         req.state = RequestState.FINISHED
         req.finish_reason = reason
+        req.finish_time = req.finish_time or time.monotonic()
         return was_live
 
     def stats(self) -> dict:

@@ -157,12 +157,14 @@ KERNEL_SIGNATURES = {
     "zk_sample": [_VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP],
     "zk_sample_cutoff": [_VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP],
     "zk_penalize": [_VP, _I, _VP, _VP, _VP, _I, _VP],
+    "zk_probe_read": [_VP, _SZ, _VP, _VP],
 }
 # present only in the bf16 library
 BF16_KERNEL_SIGNATURES = {
     "zk_gemm_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, C.c_size_t, C.POINTER(C.c_int), _VP],
     "zk_gemm_bf16_static": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
     "zk_strip_layout": [_VP, _VP, _I, _I, _VP],
+    "zk_probe_mfma_bf16": [_I, _VP, C.POINTER(C.c_double), _VP],
     "zk_qkv_rope_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "zk_attention_bf16": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
                           _F, _F, _I, _I, _VP, _SZ, _VP],
