@@ -226,7 +226,8 @@ def run_workload(name, a):
     max_len = max(lengths) + n_new
     blocks = sum(-(-(n + n_new) // page) for n in lengths) + 8
     eng = Engine(model, dtype="bfloat16", block_size=page, num_blocks=blocks, max_batch_tokens=4096,
-                 max_batch_seqs=len(prompts), prefill_chunk_size=512, max_seq_len=max_len)
+                 max_batch_seqs=len(prompts), prefill_chunk_size=512, max_seq_len=max_len,
+                 use_graphs=not a.no_graphs)
     # a small run first: code objects load, the arena and the first graphs are made
     eng.generate([p[:70] for p in prompts[:2]], SamplingParams(max_tokens=6, temperature=0.0))
     m = eng.runner.manager
@@ -289,7 +290,8 @@ def main():
     ap.add_argument("--model", choices=sorted(MODELS), default="2b", help="layer sizes: Gemma 2 2B (the default), 9B or 27B")
     ap.add_argument("--workload", choices=["9b", "27b"], default=None,
                     help="run one of the larger workloads through Engine.generate instead")
-    ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--no-graphs", action="store_true",
+                    help="decode steps run eagerly (rocprofv3's kernel trace has crashed on launches of large graphs)")
     ap.add_argument("--no-check", action="store_true", help="profiling aid: skip the check before timing")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="profiling aid: run one of the two workloads (the JSON line then lacks the other)")
