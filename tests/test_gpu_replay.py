@@ -264,3 +264,58 @@ def test_a_decoded_tokens_bits_do_not_depend_on_the_batch_in_bfloat16(tmp_path):
     small.step([StepEntry("main", main[:150], [])])
     z = small.step([StepEntry("main", [main[150]], [0])])
     assert np.abs(z[0] - alone_graph[0]).max() < 0.02 * np.abs(alone_graph[0]).max()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_launched_from_their_written_down_lists(cases, dtype):
+    """An eager step whose shape was seen before is launched by the native side from the list
+    written down the first time.  Other tokens, other positions, other pages, the same shape:
+    the logits equal, bit for bit, those of a runner that launches every kernel from Python."""
+    name = "B"
+    folder, streams, refs = cases[(name, dtype)]
+    reqs = ["r0", "r1", "r4"]
+    sub = {r: streams[r] for r in reqs}
+    # portions of equal sizes for different requests, then single tokens side by side: many repeats
+    steps = [([("r0", 8)], []), ([("r1", 8)], []), ([("r4", 8)], []), ([("r0", 8), ("r1", 8)], []),
+             ([("r4", 8), ("r0", 8)], []), ([("r1", 3), ("r4", 1)], []), ([("r0", 3), ("r1", 1)], [])]
+    steps += [([("r0", 1), ("r1", 1), ("r4", 1)], []) for _ in range(12)]
+
+    def run(lists):
+        runner = make_runner(folder, dtype, page_size=8, cache_tokens=512, max_seqs=4, max_batch_tokens=64,
+                             max_model_len=256, use_steplists=lists)
+        rows = run_steps(runner, sub, steps)
+        for r in reqs:
+            runner.finish(r)
+        return rows, runner
+
+    plain_rows, plain_runner = run(False)
+    listed_rows, runner = run(True)
+    assert plain_runner.steplist_runs == 0 and not plain_runner.steplists
+    assert runner.use_steplists and runner.steplist_runs >= 12 and 0 < len(runner.steplists) <= 8
+    assert all(runner.k.steplist_size(h) > 10 for h in runner.steplists.values())
+    for r in reqs:
+        assert np.array_equal(listed_rows[r], plain_rows[r]), r
+        n = len(listed_rows[r])
+        assert_close(listed_rows[r], refs[r][:n], dtype, f"listed {r}")
+
+
+def test_a_tensor_dropped_during_capture_is_freed_after_it():
+    """Freeing device memory synchronizes, which a capturing stream does not allow; the garbage
+    collector may drop a tensor at any moment, also in the middle of a capture.  Such frees wait
+    for the end of the capture, and the captured graph still runs."""
+    from zse_amd.runtime.device import Runtime
+    rt = Runtime.get()
+    k = rt.kernels("float32")
+    doomed, pinned = rt.empty((4096,), "float32"), rt.pinned(4096)
+    target = rt.upload(np.ones(1024, np.float32))
+    rt.sync()
+    rt.capture_begin()
+    k.zk_zero(target.ptr, 4096, rt.stream)
+    del doomed, pinned                     # their memory is given back while the stream captures
+    assert len(rt._free_later) == 2
+    graph = rt.capture_end()
+    assert rt._free_later == []
+    assert rt.download(target).all()       # captured, not run
+    rt.graph_launch(graph)
+    assert not rt.download(target).any()
+    rt.graph_destroy(graph)

@@ -16,6 +16,7 @@ HIP graph per batch size as there (model_runner.py:1806-1932).
 """
 from __future__ import annotations
 
+import weakref
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -127,7 +128,7 @@ class StepRunner:
     def __init__(self, model: Model, rt: Runtime, dtype: str, page_size: int = 16,
                  num_pages: Optional[int] = None, cache_tokens: Optional[int] = None,
                  max_seqs: int = 64, max_batch_tokens: int = 4096, max_model_len: Optional[int] = None,
-                 tuned: Optional[bool] = None, use_graphs: bool = True):
+                 tuned: Optional[bool] = None, use_graphs: bool = True, use_steplists: bool = True):
         self.model, self.rt = model, rt
         self.dtype = canonical_dtype(dtype)
         if model.loaded_dtype != self.dtype:
@@ -186,7 +187,10 @@ class StepRunner:
         self.slot_bytes = slot_bytes
         self.manager = CacheManager(groups, self.page_size, self.max_seqs, self.max_model_len, slot_bytes)
         self.state = rt.zeros((self.max_seqs, max(slot_bytes // 4, 1)), F32) if slot_bytes else None
-        self.manager.on_admit = self._clear_slot
+        # the manager tells us of every admission; a weak reference, so that runner and manager
+        # do not hold each other (a runner dropped by its owner frees its memory at once)
+        me = weakref.ref(self)
+        self.manager.on_admit = lambda req, slot: me() is not None and me()._clear_slot(req, slot)
 
         # ---- step buffers
         self.arena = Arena(rt)
@@ -218,6 +222,13 @@ class StepRunner:
         # take what changes from step to step (tokens, positions, tables, slots) from device
         # memory alone.  The built-in parts do; a part says so with ``graph_safe = True``.
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in model.parts())
+        # Eager steps (prompt portions, mixed batches): the first step of a shape runs call by
+        # call and its launches are written down on the native side; later steps of that shape
+        # are launched from there with one call (zk_steplist_run).  The same condition as for
+        # graphs: what differs between steps of one shape must come from device memory.
+        self.use_steplists = bool(use_steplists) and self.graph_safe
+        self.steplists: Dict[tuple, int] = {}        # shape of a step -> handle of its launch list
+        self.steplist_runs = 0
         self.graph_logits: Optional[Tensor] = None
         self.steps_run = 0
 
@@ -298,6 +309,11 @@ class StepRunner:
             host_entries.append((e.req, m.slot(e.req), start, n))
             max_q, max_ctx = max(max_q, n), max(max_ctx, start + n)
             t += n
+        # The two maxima only size the attention kernels' grids (a block past a request's own
+        # rows or keys ends at once); rounded up, steps of many lengths share one launch list.
+        if max_q > 1:
+            max_q = -(-max_q // 32) * 32
+        max_ctx = min(-(-max_ctx // 256) * 256, max(self.max_model_len, max_ctx))
         n_rows = 0
         for i, e in enumerate(entries):
             for w in e.want:
@@ -387,6 +403,38 @@ class StepRunner:
         self.rt.graph_launch(graph)
         return self.graph_logits.rows(0, n_rows)
 
+    MAX_STEPLISTS = 256
+
+    def _forward(self, ctx, n_rows: int, out: Tensor, shape: tuple) -> None:
+        """The model on an eager step.  Device addresses follow from the step's shape (the
+        arena hands out the same addresses for the same sequence of sizes, the step's arrays
+        lie at offsets fixed by the numbers of tokens and requests), so a shape that was seen
+        before is launched from its written-down list."""
+        if not self.use_steplists:
+            self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, out)
+            return
+        handle = self.steplists.get(shape)
+        if handle is not None:
+            self.k.steplist_run(handle, ctx.stream)
+            self.steplist_runs += 1
+            return
+        self.k.steplist_begin()
+        try:
+            self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, out)
+        except BaseException:
+            h = self.k.steplist_end()
+            if h is not None:
+                self.k.steplist_destroy(h)
+            raise
+        handle = self.k.steplist_end()
+        if handle is None:
+            self.use_steplists = False       # some part launches what the native side cannot repeat
+            return
+        if len(self.steplists) >= self.MAX_STEPLISTS:
+            old = next(iter(self.steplists))
+            self.k.steplist_destroy(self.steplists.pop(old))
+        self.steplists[shape] = handle
+
     def step(self, entries: Sequence[StepEntry], download: bool = True, tokens_from: Optional[int] = None):
         """Run one step.  Returns float32 logits [wanted, vocab] on the host
         (``download=False``: the device tensor, valid until the next step).
@@ -436,7 +484,7 @@ class StepRunner:
             ctx = self._context(off, T, R, host_entries, max_q, max_ctx, n_multi)
             self.arena.reset()
             out = self.logits.rows(0, n_rows)
-            self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, out)
+            self._forward(ctx, n_rows, out, (T, R, n_rows, n_multi, max_q, max_ctx, out.ptr))
         for e in entries:
             m.commit(e.req, m.computed(e.req) + len(e.tokens))
         self.steps_run += 1

@@ -26,7 +26,7 @@ CSRC = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "csrc"))
 PKG_LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "_lib"))
 ARCH = "gfx950"
 
-COMMON_KERNELS = ["elementwise.hip", "gemm_plain.hip", "attention_plain.hip", "sampling.hip", "probe.hip"]
+COMMON_KERNELS = ["elementwise.hip", "gemm_plain.hip", "attention_plain.hip", "sampling.hip", "probe.hip", "steplist.hip"]
 BF16_KERNELS = ["gemm_bf16.hip", "attention_bf16.hip"]
 
 LIBRARIES: Dict[str, dict] = {

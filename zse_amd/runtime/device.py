@@ -8,6 +8,7 @@ is no fallback: without a GPU or without the libraries, ``Runtime()`` raises.
 from __future__ import annotations
 
 import ctypes as C
+import struct as _struct
 from dataclasses import dataclass
 from typing import Dict, Optional, Sequence, Tuple
 
@@ -89,7 +90,7 @@ class Allocation:
 
     def close(self):
         if self.ptr:
-            self.rt.lib.zrt_free(C.c_void_p(self.ptr))
+            self.rt.free_device(self.ptr)
             self.rt.allocated -= self.nbytes
             self.ptr = 0
 
@@ -118,7 +119,7 @@ class PinnedBuffer:
     def close(self):
         if self.ptr:
             self.bytes = None
-            self.rt.lib.zrt_host_free(C.c_void_p(self.ptr))
+            self.rt.free_host(self.ptr)
             self.ptr = 0
 
     def __del__(self):
@@ -210,6 +211,7 @@ class KernelLibrary:
             self._dll.zk_gemm_bf16_workspace.restype = C.c_size_t
             self._dll.zk_gemm_bf16_workspace.argtypes = []
             self.zk_gemm_bf16_workspace = self._dll.zk_gemm_bf16_workspace
+        self._init_steplists()
         want = 1 if dtype == BF16 else 0
         if self._dll.zk_act_is_bf16() != want:
             raise DeviceError(f"{path} was built for the other storage type")
@@ -219,13 +221,87 @@ class KernelLibrary:
 
     def _wrap(self, name, fn):
         dll = self._dll
+        lib = self
 
         def call(*a):
             rc = fn(*a)
             if rc != 0:
                 raise DeviceError(f"{name} failed ({rc}): {dll.zk_last_error().decode()}")
+            if lib._writing is not None:
+                lib._write_down(name, fn.argtypes, a)
         call.__name__ = name
         return call
+
+    # ---- a step's launches written down on the native side, and launched again from there
+    def _init_steplists(self):
+        d = self._dll
+        d.zk_steplist_op.restype, d.zk_steplist_op.argtypes = C.c_int, [C.c_char_p]
+        d.zk_steplist_create.restype, d.zk_steplist_create.argtypes = C.c_void_p, []
+        d.zk_steplist_destroy.restype, d.zk_steplist_destroy.argtypes = None, [C.c_void_p]
+        d.zk_steplist_size.restype, d.zk_steplist_size.argtypes = C.c_int, [C.c_void_p]
+        d.zk_steplist_add.restype = C.c_int
+        d.zk_steplist_add.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_uint64), C.c_int]
+        d.zk_steplist_run.restype = C.c_int
+        d.zk_steplist_run.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_int)]
+        d.zk_steplist_name.restype, d.zk_steplist_name.argtypes = C.c_char_p, [C.c_void_p, C.c_int]
+        self._writing = None          # the list being written, while a step runs call by call
+        self._writable = True
+        self._op_ids: Dict[str, int] = {}
+
+    def steplist_begin(self) -> int:
+        """From now on every kernel call is also written into a new list (and still runs)."""
+        if self._writing is not None:
+            raise DeviceError("a step list is being written already")
+        self._writing = self._dll.zk_steplist_create()
+        self._writable = True
+        return self._writing
+
+    def steplist_end(self) -> Optional[int]:
+        """Stops writing; the list's handle, or None if some call could not be written down
+        (the list is then destroyed)."""
+        handle, self._writing = self._writing, None
+        if handle is not None and not self._writable:
+            self._dll.zk_steplist_destroy(handle)
+            return None
+        return handle
+
+    def steplist_run(self, handle: int, stream) -> None:
+        at = C.c_int(-1)
+        rc = self._dll.zk_steplist_run(handle, stream, C.byref(at))
+        if rc != 0:
+            name = self._dll.zk_steplist_name(handle, at.value).decode()
+            raise DeviceError(f"{name} (call {at.value} of a written-down step) failed ({rc}): "
+                              f"{self._dll.zk_last_error().decode()}")
+
+    def steplist_destroy(self, handle: int) -> None:
+        self._dll.zk_steplist_destroy(handle)
+
+    def steplist_size(self, handle: int) -> int:
+        return self._dll.zk_steplist_size(handle)
+
+    def _write_down(self, name, argtypes, args) -> None:
+        op = self._op_ids.get(name)
+        if op is None:
+            op = self._op_ids[name] = self._dll.zk_steplist_op(name.encode())
+        if op < 0 or not self._writable:
+            self._writable = False          # an entry point the native side cannot call again
+            return
+        words = (C.c_uint64 * len(args))()
+        for i, (t, v) in enumerate(zip(argtypes, args)):
+            if t is _F:
+                words[i] = _struct.unpack("<I", _struct.pack("<f", v))[0]
+            elif t is _I:
+                words[i] = int(v) & 0xFFFFFFFFFFFFFFFF
+            elif v is None:
+                words[i] = 0
+            elif isinstance(v, int):
+                words[i] = v
+            elif hasattr(v, "value"):
+                words[i] = int(v.value or 0)
+            else:
+                words[i] = 1                # a by-reference output: the native side brings its own
+        if self._dll.zk_steplist_add(self._writing, op, words, len(args)) != 0:
+            self._writable = False
 
 
 class Runtime:
@@ -273,6 +349,8 @@ class Runtime:
         self.device = device
         self._check(self.lib.zrt_init(C.c_int(device)), "init")
         self.allocated = 0
+        self._capturing = False
+        self._free_later = []
         self._kernels: Dict[str, KernelLibrary] = {}
         s = C.c_void_p()
         self._check(self.lib.zrt_stream_create(C.byref(s)), "stream create")
@@ -388,13 +466,36 @@ class Runtime:
         self._check(self.lib.zrt_event_elapsed_ms(a, b, C.byref(ms)), "event elapsed")
         return ms.value
 
+    def free_device(self, ptr: int) -> None:
+        """Frees a device allocation; while a graph is being captured the free waits until the
+        capture has ended (freeing synchronizes, which a capturing stream does not allow, and
+        the garbage collector may drop a tensor at any moment)."""
+        if self._capturing:
+            self._free_later.append(ptr)
+        else:
+            self.lib.zrt_free(C.c_void_p(ptr))
+
+    def free_host(self, ptr: int) -> None:
+        """Frees page-locked host memory, after a capture in progress has ended."""
+        if self._capturing:
+            self._free_later.append(-ptr)
+        else:
+            self.lib.zrt_host_free(C.c_void_p(ptr))
+
     # -- graphs
     def capture_begin(self):
         self._check(self.lib.zrt_capture_begin(self.stream), "capture begin")
+        self._capturing = True
 
     def capture_end(self) -> int:
         g = C.c_void_p()
-        self._check(self.lib.zrt_capture_end(self.stream, C.byref(g)), "capture end")
+        try:
+            self._check(self.lib.zrt_capture_end(self.stream, C.byref(g)), "capture end")
+        finally:
+            self._capturing = False
+            pending, self._free_later = self._free_later, []
+            for p in pending:           # device pointers as they are, host pointers negated
+                (self.lib.zrt_free if p > 0 else self.lib.zrt_host_free)(C.c_void_p(abs(p)))
         return g.value
 
     def graph_launch(self, g: int):
