@@ -9,8 +9,8 @@
 //    needed.  Partial sums of the waves meet in LDS.
 //  * mid (17 <= M <= 64, strip layout): four strips a block, the activations of a k chunk
 //    shared through LDS, K split over blocks when N alone gives too few of them.
-//  * tile (M > 64, prefill): 128x256x64 (eight waves) or 128x128x64 (four) block tiles staged
-//    through LDS, each wave a 64x64 corner built from 32x32x16 MFMAs.
+//  * tile (M > 64, prefill): 256x256x64 (sixteen waves), 128x256x64 (eight) or 128x128x64 (four)
+//    block tiles staged through LDS, each wave a 64x64 corner built from 32x32x16 MFMAs.
 // Epilogues: plain store (bf16 or float), soft cap on float output (LM head), and
 // the gated activation act(gate) * up over a [2I, K] weight whose first I rows are
 // the gate (the feed-forward's first product; the [T, 2I] intermediate never
@@ -948,6 +948,19 @@ static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc
 #define ZK_TILE(W_, M_, N_)                                                                            \
   (gated ? (exact ? ZK_TILE_(W_, M_, N_, true, true) : ZK_TILE_(W_, M_, N_, true, false))             \
          : (exact ? ZK_TILE_(W_, M_, N_, false, true) : ZK_TILE_(W_, M_, N_, false, false)))
+  // 256 x 256 blocks of sixteen waves where there are tiles enough.  The tile product is bound
+  // by what L2 delivers to a CU (a 128 x 256 x 64 step moves 48 KB for 4.2 MFLOP: at the 10 TB/s
+  // all CUs get together that is 0.9 PFLOP/s, which is what the 128 x 256 blocks reach); a
+  // 256 x 256 block moves a third fewer bytes per flop.  Measured against 128 x 256: 0.88 of its
+  // time with many rounds of tiles (4096 x 36864 x 4608 gated), 0.91 at 2048 x 9216 x 2304 gated
+  // (2.25 rounds), 1.4 at 2048 x 4096 x 2304 (half a round: half of the CUs idle).  The rule:
+  // time = (rounds, at least one, + 0.15) x time of a tile.
+  if (wide && exact) {
+    const long nb_big = (long)((M + 255) / 256) * ((N + (gated ? 128 : 256) - 1) / (gated ? 128 : 256));
+    auto rounds_cost = [](long nb, double unit) { return ((nb > 256 ? nb / 256.0 : 1.0) + 0.15) * unit; };
+    if (rounds_cost(nb_big, 2.0 * 0.8836 * 32768.0 / 1.2) < rounds_cost(nb_wide, 32768.0 / 1.2))
+      return gated ? ZK_TILE_(2, 4, 4, true, true) : ZK_TILE_(2, 4, 4, false, true);
+  }
   if (wide) return ZK_TILE(2, 2, 4);
   if (low) return ZK_TILE(1, 2, 2);
   return ZK_TILE(2, 2, 2);
