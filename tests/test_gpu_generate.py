@@ -301,3 +301,52 @@ def test_bfloat16_generation_with_preemption_and_runs_of_steps(tiny_folders):
             assert z[-1] - z[-2] < 0.05, f"prompt {p}: token {i} differs at a margin of {z[-1] - z[-2]:.3f}"
             break                      # the two runs follow different tokens from here on
     assert checked > 24 * len(prompts) * 0.8
+
+
+def test_zse_generate_with_random_weights_made_on_the_device(tmp_path):
+    """``zse generate --random-weights`` needs a folder with a config.json only; the weights it
+    draws on the device are those ``write_random_model`` writes for the same seed."""
+    import json
+    from zse_amd.engine.engine import Engine
+    from zse_amd.sampling import SamplingParams
+    from zse_amd.weights import write_random_model
+    cfg = TINY["A"][0]
+    bare = tmp_path / "bare"
+    bare.mkdir()
+    (bare / "config.json").write_text(json.dumps(cfg))
+    prompt = random_tokens(512, 9, 77)
+    p = subprocess.run([sys.executable, "-m", "zse_amd", "generate", str(bare), "--random-weights", "--weight-seed", "3",
+                        "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "6", "--temperature", "0",
+                        "--dtype", "float32", "--block-size", "4", "--num-blocks", "32", "--max-seq-len", "64", "-q"],
+                       capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    got = list(map(int, p.stdout.split()))
+    folder = write_random_model(str(tmp_path / "written"), cfg, seed=3, dtype="float32")
+    eng = Engine(folder, dtype="float32", block_size=4, num_blocks=32, max_seq_len=64)
+    assert got == eng.generate([prompt], SamplingParams(max_tokens=6, temperature=0.0))[0]
+    eng.close()
+
+
+def test_the_windowed_group_gets_a_pool_of_its_own_size(tiny_folders):
+    """Sliding layers never hold more than their window and one step's tokens per request, so
+    the engine gives their group a small pool; requests far longer than the window run on it
+    (pages are handed back as the window passes them) and give the plain implementation's tokens."""
+    from zse_amd.engine.engine import Engine
+    from zse_amd.sampling import SamplingParams
+    cfg = TINY["A"][0]                                   # window 8
+    folder = tiny_folders[("A", "float32")]
+    w = read_weights(folder)
+    eng = Engine(folder, dtype="float32", block_size=4, num_blocks=64, max_batch_tokens=32, max_batch_seqs=2,
+                 prefill_chunk_size=4, max_seq_len=128)
+    m = eng.runner.manager
+    assert [g.window for g in m.groups] == [8, None]
+    assert [p.num_pages for p in m.pools] == [2 * (-(-(8 + 4) // 4) + 2), 64]       # 10 pages against 64
+    prompts = [random_tokens(512, n, 300 + n) for n in (41, 33)]
+    got = eng.generate(prompts, SamplingParams(max_tokens=20, temperature=0.0))
+    st = eng.stats()
+    assert st.preemptions == 0 and st.peak_pages[0] <= 10 and st.peak_pages[1] >= 2 * 13
+    assert len(st.ttft_ms) == 2 and all(t > 0 for t in st.ttft_ms) and all(t > 0 for t in st.tpot_ms)
+    assert set(st.by_kind) <= {"prefill", "mixed", "decode"} and sum(v[0] for v in st.by_kind.values()) == st.steps
+    for p, g in zip(prompts, got):
+        assert g == plain_greedy(cfg, w, p, 20)
+    eng.close()

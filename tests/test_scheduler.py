@@ -239,3 +239,23 @@ def test_penalty_counts_follow_the_continuous_batching_engine():
     assert r.penalty_counts() == {5: 1, 9: 1}                # prompt tokens count once each
     r.output_tokens += [9, 4, 4, 4]
     assert r.penalty_counts() == {5: 1, 9: 2, 4: 3}          # produced tokens add up
+
+
+def test_a_small_windowed_pool_is_what_runs_out():
+    # the windowed group has a pool of its own, sized for its window and a step's tokens: when
+    # it is the one that cannot give a page, the newest request gives way as with any pool
+    m = CacheManager([GroupInfo(8, [0], 7), GroupInfo(None, [1], 64)], 4, 4, 512)
+    s = Scheduler(SchedulerConfig(64, 8, 4), m)
+    rs = [req(i, 14, 12) for i in range(3)]          # each holds up to ceil((8 + 8) / 4) + 1 = 5 windowed pages
+    for r in rs:
+        s.add_request(r)
+    seen = False
+    for _ in range(300):
+        if not s.has_work():
+            break
+        plan, _ = run_step(s)
+        seen = seen or bool(plan.preempted)
+        assert m.pools[0].used_pages <= 7
+        m.check()
+    assert seen and not s.has_work() and all(len(r.output_tokens) == 12 for r in rs)
+    assert all(p.free_pages == p.num_pages for p in m.pools)

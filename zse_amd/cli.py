@@ -1,4 +1,4 @@
-"""Command line: ``zse generate``, ``zse replay``, ``zse info``, ``zse version``,
+"""Command line: ``zse generate``, ``zse replay``, ``zse bench``, ``zse info``, ``zse version``,
 ``zse random-weights``, ``zse build``.
 
 The reference's ``zse`` has ``serve``, ``convert``, ``info``, ``version``,
@@ -38,12 +38,11 @@ def _cmd_generate(a):
         return 2
     model = a.model
     if a.random_weights:
-        import tempfile
+        # the weights are drawn on the device, in place: nothing is written (a folder made by
+        # ``zse random-weights`` from the same config and seed holds the same values)
         from .config.base import read_config_json
-        from .weights.random_init import write_random_model
-        cfg = read_config_json(a.model)
-        model = tempfile.mkdtemp(prefix="zse_random_")
-        write_random_model(model, cfg, seed=a.weight_seed, dtype="bfloat16" if a.dtype.startswith("b") else "float32")
+        from .engine.loading import random_model
+        model = random_model(read_config_json(a.model), a.dtype, seed=a.weight_seed)
     eng = Engine(model, dtype=a.dtype, block_size=a.block_size, num_blocks=a.num_blocks,
                  max_batch_tokens=a.max_batch_tokens, max_batch_seqs=a.max_batch_seqs,
                  prefill_chunk_size=a.prefill_chunk_size, max_seq_len=a.max_seq_len, quiet=a.quiet)
@@ -67,6 +66,19 @@ def _cmd_replay(a):
     if a.trace:
         sys.stdin = open(a.trace)
     return replay_main(argv)
+
+
+def _cmd_bench(a, rest):
+    """The measurement harness: ``bench.py`` beside the package, with its own options."""
+    import os
+    import runpy
+    path = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "bench.py"))
+    if not os.path.isfile(path):
+        print(f"zse bench: {path} is not there (the harness ships with the source tree)", file=sys.stderr)
+        return 2
+    sys.argv = [path] + list(rest)
+    runpy.run_path(path, run_name="__main__")
+    return 0
 
 
 def _cmd_info(a):
@@ -144,7 +156,12 @@ def main(argv=None):
     w.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
 
     sub.add_parser("build", help="compile the native libraries for gfx950")
+    sub.add_parser("bench", help="decode and prefill throughput (options as bench.py's, after the command)",
+                   add_help=False)
 
+    argv = list(sys.argv[1:] if argv is None else argv)
+    if argv and argv[0] == "bench":
+        sys.exit(_cmd_bench(None, argv[1:]) or 0)
     a = ap.parse_args(argv)
     if not a.command:
         ap.print_help()
