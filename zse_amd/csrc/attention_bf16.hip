@@ -72,13 +72,36 @@ __device__ __forceinline__ float score_log2(const AttnParams& p, float dot) {
   return p.k1 * dot;
 }
 
+// Portions: which (group, KV head) a block takes.  Blocks go to the 8 XCDs in turn by their
+// number, and every XCD has an L2 of its own; blocks that read the same keys and values (those
+// of one KV head) are therefore given to as few XCDs as possible, so that what one of them has
+// fetched is in the L2 for the others instead of crossing from the memory side once per block.
+__device__ __forceinline__ void portion_block(int& bx, int& by) {
+  const int gx = gridDim.x, gy = gridDim.y;
+  bx = blockIdx.x;
+  by = blockIdx.y;
+  const int total = gx * gy;
+  if (total % 8) return;
+  const int lin = blockIdx.x + gx * blockIdx.y, xcd = lin & 7, slot = lin >> 3;
+  if (gy <= 8 && 8 % gy == 0) {            // 8 / gy XCDs a head
+    const int per = 8 / gy;
+    by = xcd % gy;
+    bx = slot * per + xcd / gy;
+  } else if (gy % 8 == 0) {                // gy / 8 heads an XCD
+    const int heads = gy / 8;
+    by = xcd + 8 * (slot % heads);
+    bx = slot / heads;
+  }
+}
+
 template <int HD16, bool SPLIT, bool PAIR>
 __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
   constexpr int DT = (HD16 + 1) / 2;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lr = lane & 31, lk = lane >> 5;
   const int r = p.r_begin + blockIdx.z;
-  const int kvh = blockIdx.y;
+  int block_x = blockIdx.x, kvh = blockIdx.y;
+  if (!SPLIT) portion_block(block_x, kvh);
   const int qs = p.q_start[r], n = p.q_start[r + 1] - qs;
   if (n <= 0) return;
   const int start = p.ctx_len[r] - n;
@@ -93,11 +116,11 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
   int na_block = 4;                                            // waves of the block's first group
   // single groups: the last group of a portion sees the most keys and goes first, so that the
   // blocks still running at the end are the short ones
-  if (!SPLIT && !PAIR) gi = (n + p.tpw - 1) / p.tpw - 1 - (int)blockIdx.x;
+  if (!SPLIT && !PAIR) gi = (n + p.tpw - 1) / p.tpw - 1 - block_x;
   if (PAIR) {
     const int groups = (n + p.tpw - 1) / p.tpw;
-    if ((int)blockIdx.x >= (groups + 1) / 2) return;           // the whole block is past the portion
-    const int ga = groups - 1 - blockIdx.x, gb = blockIdx.x;
+    if (block_x >= (groups + 1) / 2) return;           // the whole block is past the portion
+    const int ga = groups - 1 - block_x, gb = block_x;
     if (ga != gb) {
       auto tiles_of = [&](int gr) {
         const int lo = start + gr * p.tpw, hi = start + min(n, (gr + 1) * p.tpw) - 1;
@@ -113,7 +136,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
       gi = ga;
     }
   }
-  const int chunk = SPLIT ? blockIdx.x * 4 + wave : 0;
+  const int chunk = SPLIT ? block_x * 4 + wave : 0;
   const int t0 = gi * p.tpw;
   if (!PAIR && (gi < 0 || t0 >= n)) return;
   const int g = p.nh / p.nkv;
