@@ -301,6 +301,11 @@ ATT_CASES = [
     # a portion whose row groups number 280: two groups a block (144 blocks run at once)
     dict(nh=8, nkv=8, hd=16, bs=16, reqs=[(20, 1100)], window=300, cap=20.0),
     dict(nh=10, nkv=2, hd=48, bs=16, reqs=[(3, 20), (60, 1)], window=24, cap=10.0),      # plain kernel only
+    # portions whose blocks number a multiple of 8: the blocks of a KV head are dealt to 8 / nkv
+    # XCDs (4, 2 and 1 KV heads), two requests in one launch
+    dict(nh=8, nkv=4, hd=64, bs=16, reqs=[(37, 128), (0, 100)], window=0, cap=50.0),
+    dict(nh=4, nkv=2, hd=32, bs=16, reqs=[(11, 64), (70, 50)], window=40, cap=0.0),
+    dict(nh=2, nkv=1, hd=128, bs=16, reqs=[(5, 256)], window=0, cap=30.0),
 ]
 
 
