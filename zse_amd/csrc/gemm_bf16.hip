@@ -973,6 +973,32 @@ extern "C" int zk_strip_layout(const void* src, void* dst, int N, int K, void* s
 // rounded to 16 bits (zk_norm_add_norm reads them so), before the next product overwrites them.
 extern "C" size_t zk_gemm_bf16_workspace() { return ZK_GEMM_WORKSPACE_BYTES; }
 
+// A tile variant (0: 128 x 128 blocks of four waves, 1: 64 x 128, 2: 128 x 256 of eight,
+// 3: 256 x 256 of sixteen) with K split into ks ranges, and a model of its time in microseconds:
+// the CU with the most blocks works through them one after the other, a block costs a start-up
+// and a time per 64-wide k tile, a lone block a CU differs from one of several by a factor,
+// and a split adds a joining kernel that moves the partial sums.  The constants are fitted to
+// measurements (see where it is used).
+struct TileChoice { int v, ks; };
+static double tile_cost(TileChoice c, int M, int N, int K, bool gated, size_t room) {
+  static const int BM[4] = {128, 64, 128, 256}, BN[4] = {128, 128, 256, 256};
+  static const double start[4] = {0.0, 0.0, 0.974, 4.75}, per_ktile[4] = {0.522, 0.344, 0.881, 1.48},
+                      lone[4] = {1.274, 1.432, 0.994, 0.903};
+  const double launch = 3.774, join_start = 4.183, join_per_mb = 0.553;
+  const int ncols = gated ? BN[c.v] / 2 : BN[c.v];
+  const long tiles = (long)((M + BM[c.v] - 1) / BM[c.v]) * ((N + ncols - 1) / ncols);
+  const double range_bytes = (double)tiles * BM[c.v] * BN[c.v] * 4.0;
+  int ks = c.ks;
+  while (ks > 1 && range_bytes * ks > (double)room) ks--;     // as the launcher will clamp it
+  if (ks != c.ks) return 1e30;                                  // priced under the split it becomes
+  if (ks > 1 && (K + GT_BK - 1) / GT_BK < 2 * ks) return 1e30;  // no ranges of less than two k tiles
+  const int ktiles = ((K + GT_BK - 1) / GT_BK + ks - 1) / ks;
+  const long per_cu = (tiles * ks + 255) / 256;
+  double t = launch + per_cu * (start[c.v] + ktiles * per_ktile[c.v]) * (per_cu == 1 ? lone[c.v] : 1.0);
+  if (ks > 1) t += join_start + ks * range_bytes / 1e6 * join_per_mb;
+  return t;
+}
+
 static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
                          int M, int N, int K, int epi, float cap, int w_strip, const GemmWorkspace& wsp,
                          int* parts, void* stream) {
@@ -1032,14 +1058,37 @@ static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc
   // time with many rounds of tiles (4096 x 36864 x 4608 gated), 0.91 at 2048 x 9216 x 2304 gated
   // (2.25 rounds), 1.4 at 2048 x 4096 x 2304 (half a round: half of the CUs idle).  The rule:
   // time = (rounds, at least one, + 0.15) x time of a tile.
+  int variant = wide ? 2 : low ? 1 : 0;       // 128 x 128, 64 x 128, 128 x 256, 256 x 256
   if (wide && exact) {
     const long nb_big = (long)((M + 255) / 256) * ((N + (gated ? 128 : 256) - 1) / (gated ? 128 : 256));
     auto rounds_cost = [](long nb, double unit) { return ((nb > 256 ? nb / 256.0 : 1.0) + 0.15) * unit; };
-    if (rounds_cost(nb_big, 2.0 * 0.8836 * 32768.0 / 1.2) < rounds_cost(nb_wide, 32768.0 / 1.2))
-      return gated ? ZK_TILE_(2, 4, 4, true, true) : ZK_TILE_(2, 4, 4, false, true);
+    if (rounds_cost(nb_big, 2.0 * 0.8836 * 32768.0 / 1.2) < rounds_cost(nb_wide, 32768.0 / 1.2)) variant = 3;
   }
-  if (wide) return ZK_TILE(2, 2, 4);
-  if (low) return ZK_TILE(1, 2, 2);
+  // The rules above are right for the shapes they were made on and miss elsewhere: long K with
+  // few hundred rows wants more ranges of K than they allow, narrow products of thousands of
+  // rows (N = 2304 to 4608) the 256 x 256 blocks.  So every variant and split is priced by a
+  // model of its time fitted to a sweep of 1339 measured (rows, shape, variant, split)
+  // combinations (2B, 9B and 27B layer shapes, 96 to 4096 rows; 10 % rms error), and the model's
+  // choice replaces the rules' when it promises at least 12 % (with that margin it was never
+  // more than 3 % slower than the rules on the sweep, and 5 % faster in the sum).
+  {
+    const TileChoice rule{variant, ksplit};
+    const size_t room = (wsp.ptr != nullptr && (uintptr_t)wsp.ptr % 64 == 0) ? wsp.split_bytes() : 0;
+    const double rule_cost = tile_cost(rule, M, N, K, gated, room);
+    TileChoice best = rule;
+    double best_cost = rule_cost;
+    static const int splits[] = {1, 2, 3, 4, 6, 8};
+    for (int v = 0; v < (exact ? 4 : 3); v++)
+      for (int ks : splits) {
+        const TileChoice c{v, ks};
+        const double t = tile_cost(c, M, N, K, gated, room);
+        if (t < best_cost) { best = c; best_cost = t; }
+      }
+    if (best_cost * 1.12 < rule_cost) { variant = best.v; ksplit = best.ks; }
+  }
+  if (variant == 3) return gated ? ZK_TILE_(2, 4, 4, true, true) : ZK_TILE_(2, 4, 4, false, true);
+  if (variant == 2) return ZK_TILE(2, 2, 4);
+  if (variant == 1) return ZK_TILE(1, 2, 2);
   return ZK_TILE(2, 2, 2);
 #undef ZK_TILE
 #undef ZK_TILE_
