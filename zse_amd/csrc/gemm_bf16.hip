@@ -996,7 +996,13 @@ static double tile_cost(TileChoice c, int M, int N, int K, bool gated, size_t ro
   const long per_cu = (tiles * ks + 255) / 256;
   double t = launch + per_cu * (start[c.v] + ktiles * per_ktile[c.v]) * (per_cu == 1 ? lone[c.v] : 1.0);
   if (ks > 1) t += join_start + ks * range_bytes / 1e6 * join_per_mb;
-  return t;
+  // No faster than memory delivers: the blocks of a weight tile's column walk through all of
+  // the activations, which come from memory once per column when they are too many to stay in
+  // the memory-side cache (4096 rows of K = 36864: 302 MB, 36 columns of 128: 11 GB).
+  const double a_mb = (double)M * K * 2.0 / 1e6, w_mb = (gated ? 2.0 : 1.0) * N * K * 2.0 / 1e6;
+  const double traffic_mb = w_mb + a_mb * (a_mb > 128.0 ? (double)((N + ncols - 1) / ncols) : 1.0);
+  const double memory = traffic_mb / 6.0;          // 6 TB/s
+  return t > memory ? t : memory;
 }
 
 static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
