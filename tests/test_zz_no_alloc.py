@@ -86,11 +86,11 @@ def test_static_product_equals_the_one_with_a_workspace(rt, dll):
     assert dll.zk_gemm_bf16_static_init() == 0, dll.zk_last_error().decode()
     assert dll.zk_gemm_bf16_static_init() == 0           # a second set-up call changes nothing
     ws = rt.zeros((rt.kernels("bfloat16").zk_gemm_bf16_workspace() // 4,), "float32")
-    # 40 rows, N = 2304: 36 column blocks, so K is split into 7 ranges whose partial sums
-    # (7 planes of [40, 2304] floats, 2.6 MB) go through the static array
+    # 40 rows, N = 2304: 36 column blocks, so K is split into ranges whose partial sums
+    # (planes of [40, 2304] floats, 0.37 MB each) go through the static array
     g, w = both(rt, dll, ws, 40, 2304, 2304, seed=1)
     assert np.array_equal(g, w)
-    assert ranges_of(rt, dll, ws, 40, 2304, 2304) == 7     # the shape does go through the scratch memory
+    assert ranges_of(rt, dll, ws, 40, 2304, 2304) >= 2     # the shape does go through the scratch memory
     # the second call is smaller: other plane sizes, over what the first call left behind
     g, w = both(rt, dll, ws, 24, 1152, 1024, seed=2)
     assert np.array_equal(g, w)

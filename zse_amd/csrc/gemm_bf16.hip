@@ -840,11 +840,19 @@ static int launch_mid(const void* A, int lda, const void* W, void* C, int ldc, i
   const int mt = (M + 15) / 16;
   const int npad = (N + 15) / 16 * 16;
   const int cblocks = ((N + 15) / 16 + 3) / 4;
-  // split K until every CU has a block, a range no shorter than a chunk; more ranges than that
-  // cost more in partial sums than they gain (measured at N = 2304 and 4096, M = 32 and 64)
-  int ksplit = 256 / cblocks;
-  if (ksplit > K / 32 / GM_STEPS) ksplit = K / 32 / GM_STEPS;
-  if (ksplit < 1) ksplit = 1;
+  // Split K until every CU has a block, a range no shorter than a chunk of GM_STEPS steps; two
+  // blocks a CU where ranges stay long (16 chunks or more: the blocks of a CU then cover each
+  // other's waits).  More ranges than that cost more in partial sums than they gain.  The
+  // longest range sets the time, so of the splits with that longest range the one with the
+  // fewest ranges is taken (8 chunks: 4 ranges of 2 instead of 7 of 1 or 2; measured at the
+  // shapes of the 2B, 9B and 27B layers with 24 to 64 rows).
+  const int chunks = max(1, K / 32 / GM_STEPS);
+  int ksplit = max(1, min(256 / cblocks, chunks));
+  if (chunks / max(1, 512 / cblocks) >= 16) ksplit = max(1, min(512 / cblocks, chunks));
+  {
+    const int longest = (chunks + ksplit - 1) / ksplit;
+    ksplit = (chunks + longest - 1) / longest;
+  }
   const size_t per_range = (size_t)(GATED ? 2 : 1) * M * npad * sizeof(float);
   void* ws = wsp.ptr;
   if (ws == nullptr || (uintptr_t)ws % 16 != 0) ksplit = 1;
