@@ -160,6 +160,33 @@ def test_gemm_bf16_strip_layout(rt, M, N, K, gated):
         assert np.array_equal(rt.download(out), w[toks] * np.float32(2.0))
 
 
+@pytest.mark.parametrize("N,K,gated", [(2304, 9216, False), (4096, 2304, False), (9216, 2304, True), (4608, 4096, False)])
+def test_gemm_bf16_layer_shapes_at_medium_rows(rt, N, K, gated):
+    """Layer-size products with a hundred to a thousand rows, where the dispatch picks among four
+    tile sizes and up to eight ranges of K by a model of their times: whatever it picks agrees
+    with the plain product of the same library (same 16-bit inputs, float sums)."""
+    k = rt.kernels("bfloat16")
+    rng = np.random.default_rng(N + K)
+    rows = 2 * N if gated else N
+    w = bf16(rng.normal(size=(rows, K)) * (0.02 if gated else 0.05))
+    W = up(rt, w, "bfloat16")
+    WS = rt.empty((rows, K), "bfloat16")
+    k.zk_strip_layout(W.ptr, WS.ptr, rows, K, rt.stream)
+    ws = gemm_workspace(rt)
+    for M in (96, 200, 384, 520, 1000):
+        a = bf16(rng.normal(size=(M, K)))
+        A = up(rt, a, "bfloat16")
+        C, R = rt.empty((M, N), "float32"), rt.empty((M, rows), "float32")
+        k.zk_gemm_bf16(A.ptr, K, WS.ptr, C.ptr, N, 1, M, N, K, 2 if gated else 0, 0.0, 1, ws.ptr, ws.nbytes,
+                       None, rt.stream)
+        k.zk_gemm_plain(A.ptr, K, W.ptr, R.ptr, rows, 1, M, rows, K, rt.stream)
+        got, ref = rt.download(C), rt.download(R).astype(np.float64)
+        want = gelu(ref[:, :N]) * ref[:, N:] if gated else ref
+        tol = 2e-5 * math.sqrt(K) * max(1.0, np.abs(want).max())
+        err = np.abs(got - want).max()
+        assert err < tol, f"M={M}: {err} against {tol}"
+
+
 def test_gemm_bf16_random_shapes(rt):
     """Forty shapes drawn at random over the three kernels' ranges, both weight layouts, with
     and without the gated epilogue and the workspace: whatever the dispatch picks must agree
