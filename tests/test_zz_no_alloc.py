@@ -82,7 +82,7 @@ def ranges_of(rt, dll, ws, M, N, K):
 
 
 def test_static_product_equals_the_one_with_a_workspace(rt, dll):
-    assert dll.zk_gemm_bf16_static_bytes() == 8 << 20
+    assert dll.zk_gemm_bf16_static_bytes() == 16 << 20
     assert dll.zk_gemm_bf16_static_init() == 0, dll.zk_last_error().decode()
     assert dll.zk_gemm_bf16_static_init() == 0           # a second set-up call changes nothing
     ws = rt.zeros((rt.kernels("bfloat16").zk_gemm_bf16_workspace() // 4,), "float32")
@@ -106,14 +106,15 @@ def test_static_product_equals_the_one_with_a_workspace(rt, dll):
 
 
 def test_static_product_refuses_what_does_not_fit(rt, dll):
-    # 1024 rows, N = 1024, K = 16384: 64 tiles of 128 x 128 split K into 4 ranges, 16 MB of
-    # partial sums; the array holds 8 MB, so the call is refused and nothing is launched
-    M, N, K = 1024, 1024, 16384
+    # 1024 rows, N = 1024, K = 65536: a few dozen tiles and a very long K, so K is split into
+    # eight ranges, 32 MB of partial sums; the array holds 16 MB, so the call is refused and
+    # nothing is launched
+    M, N, K = 1024, 1024, 65536
     A = rt.zeros((M, K), "bfloat16")
     W = rt.zeros((N, K), "bfloat16")
     out = rt.zeros((M, N), "bfloat16")
     rc = dll.zk_gemm_bf16_static(A.ptr, K, W.ptr, out.ptr, N, 0, M, N, K, 0, 0.0, 0, rt.stream)
     assert rc != 0
     msg = dll.zk_last_error().decode()
-    assert "static scratch array holds 8388608" in msg and "need" in msg
+    assert "static scratch array holds 16777216" in msg and "need" in msg
     rt.sync()

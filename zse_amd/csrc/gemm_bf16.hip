@@ -27,7 +27,7 @@
 // Where a product that splits K over blocks leaves its partial sums.  ``strict``: the split is
 // chosen as for the standard workspace (so that the bits do not depend on who brought the
 // memory) and refused, not narrowed, when ``bytes`` cannot hold it.
-#define ZK_GEMM_WORKSPACE_BYTES ((size_t)64 << 20)
+#define ZK_GEMM_WORKSPACE_BYTES ((size_t)320 << 20)
 struct GemmWorkspace {
   void* ptr;
   size_t bytes;

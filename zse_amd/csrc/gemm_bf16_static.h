@@ -12,8 +12,10 @@
 //  * K is split exactly as zk_gemm_bf16 splits it with its standard workspace
 //    (zk_gemm_bf16_workspace() bytes), so both give the same bits.  A shape whose partial sums
 //    do not fit the array is refused with an error that names both sizes; nothing is launched.
-//    Products of up to 64 rows always fit; products of more rows that split K fit while
-//    (blocks of 128 x 128) x (ranges of K) x 64 KB stays within the array.
+//    Products of up to 64 rows always fit (their ranges times their padded width stay within
+//    32768 columns: 64 x 32768 floats, twice that with a gate, are the array's 16 MiB);
+//    products of more rows that split K fit while (tiles) x (ranges of K) x (4 bytes a tile
+//    element) stays within the array.
 //  * Every call on a GPU shares that GPU's array, which keeps the last call's contents.
 //    Nothing in it has to start at zero (each plane of partial sums is written in full before
 //    it is read, within one call), so calls need no clearing between them; but two calls
@@ -25,7 +27,7 @@
 #pragma once
 #include <cstddef>
 
-#define ZK_GEMM_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
+#define ZK_GEMM_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
 
 extern "C" {
 
