@@ -223,7 +223,9 @@ def test_gemm_bf16_random_shapes(rt):
 
 
 @pytest.mark.parametrize("M,N,K", [(8, 2304, 2048), (1, 2304, 9216), (16, 1024, 4096), (40, 2304, 9216), (64, 4096, 2304),
-                                   (17, 1536, 1024)])
+                                   (17, 1536, 1024),
+                                   # up to 16 rows and more strips than CUs, unevenly spread: K in ranges
+                                   (8, 4608, 36864), (1, 4608, 4096), (16, 5120, 2048)])
 def test_gemm_bf16_leaves_partial_sums_to_a_reader_that_asks(rt, M, N, K):
     """A caller that passes a place for the number of parts gets the split product's partial
     sums as planes of [M, N] floats; added in order and rounded they are the bits the product
@@ -247,6 +249,8 @@ def test_gemm_bf16_leaves_partial_sums_to_a_reader_that_asks(rt, M, N, K):
     k.zk_gemm_bf16(A.ptr, K, WS.ptr, C2.ptr, N, 0, M, N, K, 0, 0.0, 1, ws.ptr, ws.nbytes, ctypes.byref(parts), rt.stream)
     P = parts.value
     assert P >= 0
+    if M <= 16 and N > 4096:
+        assert P >= 2          # 288 and 320 strips over 256 CUs
     if P == 0:
         assert np.array_equal(rt.download_f32(C2), joined)
         return

@@ -102,12 +102,13 @@ __device__ __forceinline__ void store4(__bf16* dst, const float (&x)[4]) {
 // alone: with loads under per-lane conditions it waits for every load before each group, and
 // the next group's loads, just issued, no longer overlap anything (down projection of 2304 x
 // 9216 at 8 rows: 14 us against 9).
-template <int MT, bool GATED, int NW, bool ROPE = false, bool EXACT = false>
+template <int MT, bool GATED, int NW, bool ROPE = false, bool EXACT = false, bool SPLIT = false>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __restrict__ A, int lda,
                                                           const __bf16* __restrict__ W,
                                                           void* __restrict__ C, int ldc, int c_is_f32,
                                                           int M, int N, int K, int epi, float cap,
-                                                          int w_strip, RopeStore rs) {
+                                                          int w_strip, RopeStore rs,
+                                                          float* __restrict__ partials = nullptr, int ksplit = 1) {
   static_assert(!ROPE || (MT == 1 && !GATED), "the rotating epilogue takes up to 16 rows");
   constexpr int NS = GATED ? 2 : 1;
   __shared__ f32x4 red[NW - 1][NS][MT][64];
@@ -160,7 +161,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
   // EXACT: whole groups of STEPS steps are shared out among the waves as evenly as they go
   const int total_groups = (total_steps + STEPS - 1) / STEPS;
   const int uwave = __builtin_amdgcn_readfirstlane(wave);      // the same in every lane: loop bounds stay scalar
-  const int gw0 = uwave * total_groups / NW, gw1 = (uwave + 1) * total_groups / NW;
+  // (SPLIT) blockIdx.y takes one of ksplit ranges of the groups, its waves share the range out
+  static_assert(!SPLIT || (EXACT && MT == 1 && !GATED && !ROPE), "K is split for plain products of up to 16 rows");
+  const int gy0 = SPLIT ? (int)blockIdx.y * total_groups / ksplit : 0;
+  const int gy1 = SPLIT ? ((int)blockIdx.y + 1) * total_groups / ksplit : total_groups;
+  const int gw0 = gy0 + uwave * (gy1 - gy0) / NW, gw1 = gy0 + (uwave + 1) * (gy1 - gy0) / NW;
   const int run_lo = gw0 * STEPS, run_n = (gw1 - gw0) * STEPS;      // the wave's run of steps
   auto fetch = [&](int s0, bf16x8 (&wf)[NS][STEPS], bf16x8 (&af)[MT][STEPS]) {
     if (EXACT) {
@@ -277,6 +282,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
       v[g] = acc[g][mt];
 #pragma unroll
       for (int w = 0; w < NW - 1; w++) v[g] += red[w][g][mt][lane];
+    }
+    if (SPLIT) {
+      // the range's partial sums: plane blockIdx.y of [M, npad] floats, to be added up in the
+      // order of the ranges by whoever reads them (zk_norm_add_norm, or the joining kernel)
+      if (m < M) {
+        const size_t npad = (size_t)gridDim.x * 16;
+        *(f32x4*)(partials + ((size_t)blockIdx.y * M + m) * npad + n0 + 4 * kq) = v[0];
+      }
+      continue;
     }
     if (ROPE) {
       // results 4 kq + i of the block's 16: lanes 0..31 hold places hpos + 4 kq + i of the
@@ -881,11 +895,41 @@ static int launch_mid(const void* A, int lda, const void* W, void* C, int ldc, i
 
 template <bool GATED>
 static int launch_skinny(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M,
-                         int N, int K, int epi, float cap, int w_strip, hipStream_t s) {
+                         int N, int K, int epi, float cap, int w_strip, const GemmWorkspace& wsp, int* parts,
+                         hipStream_t s) {
   const int mt = (M + 15) / 16;
   dim3 grid((N + 15) / 16);
+  // A strip is a block, and the blocks of a CU share its way to memory: the kernel takes as
+  // long as the CU with the most blocks.  288 strips (N = 4608) leave 32 of the 256 CUs with two
+  // blocks and the rest with one, twice the time of an even spread; 144 strips leave 112 CUs
+  // idle.  Splitting K into ks ranges makes ks times the blocks of 1/ks the length, and the time
+  // of the fullest CU goes with ceil(strips ks / 256) / ks.  That pays where strips are more
+  // than the CUs and spread unevenly (N = 4608 with K = 36864 at 8 rows: 87 -> 50 us with eight
+  // ranges); with fewer strips than CUs it was measured three times and lost each time (144
+  // strips, two and eight ranges: the product then goes as fast as memory gives to this pattern
+  // of reads whatever the number of CUs, and the shorter blocks only add their start-up).
+  // Only where the reader adds up the partial sums itself (the norm kernel, through `parts`):
+  // a joining launch would cost what the split gains.
+  int ksplit = 1;
+  float* partials = (float*)wsp.ptr;
+  const size_t npad = (size_t)grid.x * 16;
+  if (!GATED && mt == 1 && w_strip && grid.x > 256 && parts != nullptr && partials != nullptr &&
+      (uintptr_t)partials % 16 == 0 && joinable_by_reader(N, ldc, c_is_f32, epi)) {
+    auto longest = [&](int ks) { return (double)(((long)grid.x * ks + 255) / 256) / ks; };
+    double best = longest(1);
+    for (int ks = 2; ks <= 8; ks *= 2) {
+      if (K / ks < 1024 || (size_t)ks * M * npad * sizeof(float) > wsp.split_bytes()) break;
+      if (longest(ks) < 0.97 * best && longest(ks) <= 0.85 * longest(1)) {
+        best = longest(ks);
+        ksplit = ks;
+      }
+    }
+    if (ksplit > 1 && (size_t)ksplit * M * npad * sizeof(float) > wsp.bytes)
+      return wsp.too_small((size_t)ksplit * M * npad * sizeof(float));
+    grid.y = ksplit;
+  }
   // few strips: eight waves a strip keep enough loads in flight
-  const bool wide = grid.x < 512 && K >= 2048 && mt <= 2;
+  const bool wide = (long)grid.x * ksplit < 512 && K / ksplit >= 2048 && mt <= 2;
 #define ZK_SKINNY(MT_, NW_)                                                                           \
   do {                                                                                                \
     if (w_strip)                                                                                      \
@@ -895,11 +939,23 @@ static int launch_skinny(const void* A, int lda, const void* W, void* C, int ldc
       gemm_skinny_kernel<MT_, GATED, NW_><<<grid, NW_ * 64, 0, s>>>(                                  \
           (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, RopeStore{}); \
   } while (0)
-  if (mt == 1) { if (wide) ZK_SKINNY(1, 8); else ZK_SKINNY(1, 4); }
+  if (ksplit > 1) {
+    if constexpr (!GATED) {
+      if (wide)
+        gemm_skinny_kernel<1, false, 8, false, true, true><<<grid, 8 * 64, 0, s>>>(
+            (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, RopeStore{},
+            partials, ksplit);
+      else
+        gemm_skinny_kernel<1, false, 4, false, true, true><<<grid, 4 * 64, 0, s>>>(
+            (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, RopeStore{},
+            partials, ksplit);
+    }
+  } else if (mt == 1) { if (wide) ZK_SKINNY(1, 8); else ZK_SKINNY(1, 4); }
   else if (mt == 2) { if (wide) ZK_SKINNY(2, 8); else ZK_SKINNY(2, 4); }
   else if (mt == 3) ZK_SKINNY(3, 4);
   else ZK_SKINNY(4, 4);
 #undef ZK_SKINNY
+  if (ksplit > 1) *parts = ksplit;
   return zk_launch_status("zk_gemm_bf16 (skinny)");
 }
 
@@ -1032,8 +1088,8 @@ static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc
                  : launch_mid<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, wsp, parts, s);
   }
   if (M <= 64) {
-    return gated ? launch_skinny<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s)
-                 : launch_skinny<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, s);
+    return gated ? launch_skinny<true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, wsp, parts, s)
+                 : launch_skinny<false>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, wsp, parts, s);
   }
   // 128 x 128 blocks of four waves (two share a CU) or 128 x 256 blocks of eight (one a CU,
   // about 1.2 times the rate).  What counts is the CU with the most blocks; a lone small block
