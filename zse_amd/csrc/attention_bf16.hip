@@ -396,6 +396,21 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const int r = p.r_begin + blockIdx.z;
   const int kvh = blockIdx.y;
   const int chunk = blockIdx.x * 4 + wave;
+  const int* table = p.block_table + (size_t)r * p.max_blocks;
+  const int hd = p.hd, bsh = p.bs_shift, bmask = p.bs - 1, nkv = p.nkv;
+  // The pages of the chunk's (up to two) tiles are asked for before the request's length is
+  // known, beside it: where a key lies follows from the chunk alone.  A key past the context is
+  // masked below, so any page serves for it (a hole in the table reads page 0).
+  int kpage[2][2], vpage[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int k0 = chunk * p.chunk + 32 * i;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      kpage[i][t] = table[min((k0 + 16 * t + col) >> bsh, p.max_blocks - 1)];
+      vpage[i][t] = table[min((k0 + 16 * t + 4 * kq) >> bsh, p.max_blocks - 1)];
+    }
+  }
   const int n = p.q_start[r + 1] - p.q_start[r];
   if (n <= 0) return;
   const int pos = p.ctx_len[r] - 1;
@@ -407,8 +422,6 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const bool col_ok = col < g;
   const int head = kvh * g + (col_ok ? col : 0);
   const int trow = p.q_start[r];
-  const int* table = p.block_table + (size_t)r * p.max_blocks;
-  const int hd = p.hd, bsh = p.bs_shift, bmask = p.bs - 1, nkv = p.nkv;
 
   // the query operand waits in LDS (one 16-byte piece per lane and step), not in registers
   __shared__ bf16x8 sq[4][KS][64];
@@ -429,20 +442,23 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   for (int dt = 0; dt < DT; dt++) o[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
 
-  for (int key0 = (key_lo / 32) * 32; active && key0 <= key_hi; key0 += 32) {
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int key0 = chunk * p.chunk + 32 * i;
+    if (!active || 32 * i >= p.chunk || key0 > key_hi || key0 + 31 < key_lo) continue;
     bf16x8 kf[2][KS];
 #pragma unroll
     for (int t = 0; t < 2; t++) {
-      const int kk = min(key0 + 16 * t + col, key_hi);
-      const int page = max(table[kk >> bsh], 0);
+      const int kk = key0 + 16 * t + col;
+      const int page = max(kpage[i][t], 0);
       const __bf16* kr = p.kcache + ((((size_t)page * nkv + kvh) << bsh) + (kk & bmask)) * hd + kq * 8;
 #pragma unroll
       for (int ks = 0; ks < KS; ks++) kf[t][ks] = *(const bf16x8*)(kr + ks * 32);
     }
     bf16x8 vf[DT];
     {
-      const int ka = min(key0 + 4 * kq, key_hi & ~3), kb = min(key0 + 16 + 4 * kq, key_hi & ~3);
-      const int pa = max(table[ka >> bsh], 0), pb = max(table[kb >> bsh], 0);
+      const int ka = key0 + 4 * kq, kb = key0 + 16 + 4 * kq;
+      const int pa = max(vpage[i][0], 0), pb = max(vpage[i][1], 0);
       const __bf16* va_base = p.vcache + ((((size_t)pa * nkv + kvh) * hd) << bsh) + (ka & bmask);
       const __bf16* vb_base = p.vcache + ((((size_t)pb * nkv + kvh) * hd) << bsh) + (kb & bmask);
 #pragma unroll
