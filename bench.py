@@ -341,6 +341,13 @@ def main():
                         max_batch_tokens=max(a.prefill_tokens, max_b), max_model_len=longest,
                         use_graphs=not a.no_graphs)
     sampler = DeviceSampler(rt, runner.k, max_b)
+    # Steady state is what is measured.  For about a second after a process has allocated tens of
+    # GB (the cache slabs, just now) kernels that wait for memory rather than stream from it run
+    # up to 17 % slower (the o and down products of a decode step: 10.1 instead of 8.7 us; steps
+    # at batch 1 and 8 by 3 to 4 %); later steps of the same process do not, whatever was done
+    # meanwhile.  So the timed work starts two seconds after the allocations.
+    rt.sync()
+    time.sleep(2.0)
     greedy = SamplingParams(temperature=0.0)
     rng = np.random.default_rng(0)
     log(f"model ready in {time.time() - t0:.1f} s: {cfg['num_hidden_layers']} layers, "
