@@ -444,7 +444,7 @@ template <int WMT, int NWM, int NWN, bool GATED, bool EXACT>
 __global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_tile_kernel(
     const __bf16* __restrict__ A, int lda, const __bf16* __restrict__ W, void* __restrict__ C, int ldc,
     int c_is_f32, int M, int N, int K_all, int epi, float cap, int tiles_m, int tiles_n, int w_strip,
-    f32x16* __restrict__ partials, int ksplit) {
+    f32x16* __restrict__ partials, int ksplit, int tile_base) {
   constexpr int T = 64 * NWM * NWN;
   constexpr int BM = 32 * WMT * NWM, BN = 64 * NWN;
   constexpr int RPP = T / 8;                   // rows one pass of the block's threads covers
@@ -454,7 +454,7 @@ __global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_t
   typedef __bf16 (*tile_t)[GT_LD];
   const tile_t tiles = (tile_t)gt_lds;          // buffer b: A rows, then W rows, from row b (BM + BN)
   int tm, tn;
-  tile_of_block(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  tile_of_block(blockIdx.x + tile_base, tiles_m, tiles_n, tm, tn);     // a launch takes tiles [tile_base, tile_base + gridDim.x)
   const int m0 = tm * BM;
   constexpr int NCOLS = GATED ? BN / 2 : BN;         // output columns of the block
   const int n0 = tn * NCOLS;
@@ -614,15 +614,15 @@ __global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_t
 template <int WMT, int NWM, int NWN, bool GATED>
 __global__ __launch_bounds__(256) void gemm_tile_join_kernel(
     const f32x4* __restrict__ partials, int ksplit, void* __restrict__ C, int ldc, int c_is_f32, int M,
-    int N, int epi, float cap, int tiles_m, int tiles_n) {
+    int N, int epi, float cap, int tiles_m, int tiles_n, int tile_base, int tile_count) {
   constexpr int BM = 32 * WMT * NWM, BN = 64 * NWN, NW = NWM * NWN;
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   const int b = (int)(idx & 3), lane = (int)((idx >> 2) & 63);
   const int i = (int)((idx >> 8) % WMT), wave = (int)((idx >> 8) / WMT % NW);
-  const int tile = (int)((idx >> 8) / (WMT * NW));
-  if (tile >= tiles_m * tiles_n) return;
+  const int tile = (int)((idx >> 8) / (WMT * NW));      // counted from the launch's first tile, as the partial sums are
+  if (tile >= tile_count) return;
   int tm, tn;
-  tile_of_block(tile, tiles_m, tiles_n, tm, tn);
+  tile_of_block(tile + tile_base, tiles_m, tiles_n, tm, tn);
   // float4 index of (tile, range p, wave, pair member j, lane, b): an accumulator is 4 float4
   const size_t per_wave = (size_t)WMT * 2 * 64 * 4;
   const f32x4* src = partials + ((size_t)tile * ksplit * NW + wave) * per_wave + ((size_t)(i * 2) * 64 + lane) * 4 + b;
@@ -638,7 +638,7 @@ __global__ __launch_bounds__(256) void gemm_tile_join_kernel(
 template <int WMT, int NWM, int NWN, bool GATED, bool EXACT>
 static int launch_tile(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M, int N,
                        int K, int epi, float cap, int w_strip, const GemmWorkspace& wsp, int ksplit,
-                       hipStream_t s) {
+                       int tail_split, hipStream_t s) {
   constexpr int BM = 32 * WMT * NWM, BN = 64 * NWN;
   constexpr int ncols = GATED ? BN / 2 : BN;
   constexpr size_t lds = (size_t)2 * (BM + BN) * GT_LD * sizeof(__bf16);
@@ -658,12 +658,33 @@ static int launch_tile(const void* A, int lda, const void* W, void* C, int ldc, 
   if (ws == nullptr || (uintptr_t)ws % 64 != 0) ksplit = 1;
   while (ksplit > 1 && per_range * ksplit > wsp.split_bytes()) ksplit--;
   if (ksplit > 1 && per_range * ksplit > wsp.bytes) return wsp.too_small(per_range * ksplit);
-  gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT><<<dim3(tiles_m * tiles_n, ksplit), 64 * NWM * NWN, lds, s>>>(
+  const int tiles = tiles_m * tiles_n;
+  // The tail.  The CUs take the tiles in rounds (256 a round for the blocks of eight and sixteen
+  // waves, 512 for those of four, two of which share a CU), and a last round with few tiles
+  // costs a whole round's time.  Where the caller's model of the times says it pays (a long K:
+  // the partial sums of about 256 tile ranges, 16 to 67 MB, cost the same whatever K is), such
+  // a last round goes into a launch of its own that splits K into ``tail_split`` ranges, and a
+  // join of those tiles alone.
+  constexpr int round_blocks = 256 * (NWM * NWN <= 4 ? 2 : 1);
+  const int tail = tiles % round_blocks;
+  if (ksplit > 1 || tail == 0 || tiles <= round_blocks || ws == nullptr || (uintptr_t)ws % 64 != 0) tail_split = 1;
+  if (tail_split > 1 && (size_t)tail * tail_split * BM * BN * sizeof(float) > wsp.split_bytes()) tail_split = 1;
+  if (tail_split > 1 && (size_t)tail * tail_split * BM * BN * sizeof(float) > wsp.bytes)
+    return wsp.too_small((size_t)tail * tail_split * BM * BN * sizeof(float));
+  const int whole = tail_split > 1 ? tiles - tail : tiles;
+  gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT><<<dim3(whole, ksplit), 64 * NWM * NWN, lds, s>>>(
       (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, tiles_m, tiles_n, w_strip,
-      (f32x16*)ws, ksplit);
+      (f32x16*)ws, ksplit, 0);
   if (ksplit > 1)
-    gemm_tile_join_kernel<WMT, NWM, NWN, GATED><<<dim3(tiles_m * tiles_n * WMT * NWM * NWN), 256, 0, s>>>(
-        (const f32x4*)ws, ksplit, C, ldc, c_is_f32, M, N, epi, cap, tiles_m, tiles_n);
+    gemm_tile_join_kernel<WMT, NWM, NWN, GATED><<<dim3(tiles * WMT * NWM * NWN), 256, 0, s>>>(
+        (const f32x4*)ws, ksplit, C, ldc, c_is_f32, M, N, epi, cap, tiles_m, tiles_n, 0, tiles);
+  if (tail_split > 1) {
+    gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT><<<dim3(tail, tail_split), 64 * NWM * NWN, lds, s>>>(
+        (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, tiles_m, tiles_n, w_strip,
+        (f32x16*)ws, tail_split, whole);
+    gemm_tile_join_kernel<WMT, NWM, NWN, GATED><<<dim3(tail * WMT * NWM * NWN), 256, 0, s>>>(
+        (const f32x4*)ws, tail_split, C, ldc, c_is_f32, M, N, epi, cap, tiles_m, tiles_n, whole, tail);
+  }
   return zk_launch_status("zk_gemm_bf16 (tile)");
 }
 
@@ -1044,7 +1065,8 @@ extern "C" size_t zk_gemm_bf16_workspace() { return ZK_GEMM_WORKSPACE_BYTES; }
 // and a split adds a joining kernel that moves the partial sums.  The constants are fitted to
 // measurements (see where it is used).
 struct TileChoice { int v, ks; };
-static double tile_cost(TileChoice c, int M, int N, int K, bool gated, size_t room) {
+static double tile_cost(TileChoice c, int M, int N, int K, bool gated, size_t room, int* tail_split = nullptr) {
+  if (tail_split) *tail_split = 1;
   static const int BM[4] = {128, 64, 128, 256}, BN[4] = {128, 128, 256, 256};
   static const double start[4] = {0.0, 0.0, 0.974, 4.75}, per_ktile[4] = {0.522, 0.344, 0.881, 1.48},
                       lone[4] = {1.274, 1.432, 0.994, 0.903};
@@ -1056,10 +1078,29 @@ static double tile_cost(TileChoice c, int M, int N, int K, bool gated, size_t ro
   while (ks > 1 && range_bytes * ks > (double)room) ks--;     // as the launcher will clamp it
   if (ks != c.ks) return 1e30;                                  // priced under the split it becomes
   if (ks > 1 && (K + GT_BK - 1) / GT_BK < 2 * ks) return 1e30;  // no ranges of less than two k tiles
-  const int ktiles = ((K + GT_BK - 1) / GT_BK + ks - 1) / ks;
+  const int ktiles_all = (K + GT_BK - 1) / GT_BK;
+  const int ktiles = (ktiles_all + ks - 1) / ks;
   const long per_cu = (tiles * ks + 255) / 256;
   double t = launch + per_cu * (start[c.v] + ktiles * per_ktile[c.v]) * (per_cu == 1 ? lone[c.v] : 1.0);
   if (ks > 1) t += join_start + ks * range_bytes / 1e6 * join_per_mb;
+  // a last round of few tiles is launched apart with K in ranges (launch_tile has the rule)
+  const long round_blocks = c.v <= 1 ? 512 : 256, tail = tiles % round_blocks;
+  if (ks == 1 && tiles > round_blocks && tail > 0 && 2 * tail <= round_blocks && room > 0) {
+    const double tile_bytes = (double)BM[c.v] * BN[c.v] * 4.0;
+    int ts = (int)(round_blocks / tail < 8 ? round_blocks / tail : 8);
+    while (ts > 1 && (ktiles_all / ts < 4 || tail * ts * tile_bytes > (double)room)) ts--;
+    if (ts > 1) {
+      const long tail_per_cu = (tail * ts + 255) / 256;
+      const double apart =
+          launch + (double)((tiles - tail) / 256) * (start[c.v] + ktiles_all * per_ktile[c.v]) + 3.0 +
+          tail_per_cu * (start[c.v] + (ktiles_all + ts - 1) / ts * per_ktile[c.v]) * (tail_per_cu == 1 ? lone[c.v] : 1.0) +
+          join_start + ts * tail * tile_bytes / 1e6 * join_per_mb;
+      if (apart < 0.95 * t) {
+        t = apart;
+        if (tail_split) *tail_split = ts;
+      }
+    }
+  }
   // No faster than memory delivers: the blocks of a weight tile's column walk through all of
   // the activations, which come from memory once per column when they are too many to stay in
   // the memory-side cache (4096 rows of K = 36864: 302 MB, 36 columns of 128: 11 GB).
@@ -1117,7 +1158,7 @@ static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc
   const bool low = !wide && M > 64 && nb_small * ksplit <= 128;
   if (low) ksplit = ranges((long)((M + 63) / 64) * (nb_small / tiles_m));
 #define ZK_TILE_(W_, M_, N_, G_, E_) \
-  launch_tile<W_, M_, N_, G_, E_>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, wsp, ksplit, s)
+  launch_tile<W_, M_, N_, G_, E_>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, wsp, ksplit, tail_split, s)
 #define ZK_TILE(W_, M_, N_)                                                                            \
   (gated ? (exact ? ZK_TILE_(W_, M_, N_, true, true) : ZK_TILE_(W_, M_, N_, true, false))             \
          : (exact ? ZK_TILE_(W_, M_, N_, false, true) : ZK_TILE_(W_, M_, N_, false, false)))
@@ -1155,6 +1196,11 @@ static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc
         if (t < best_cost) { best = c; best_cost = t; }
       }
     if (best_cost * 1.12 < rule_cost) { variant = best.v; ksplit = best.ks; }
+  }
+  int tail_split = 1;
+  {
+    const size_t room = (wsp.ptr != nullptr && (uintptr_t)wsp.ptr % 64 == 0) ? wsp.split_bytes() : 0;
+    tile_cost(TileChoice{variant, ksplit}, M, N, K, gated, room, &tail_split);
   }
   if (variant == 3) return gated ? ZK_TILE_(2, 4, 4, true, true) : ZK_TILE_(2, 4, 4, false, true);
   if (variant == 2) return ZK_TILE(2, 2, 4);
