@@ -95,7 +95,7 @@ __device__ __forceinline__ void portion_block(int& bx, int& by) {
 }
 
 template <int HD16, bool SPLIT, bool PAIR>
-__global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, (HD16 <= 8 && !PAIR) ? 2 : 1) void attn_mfma_kernel(AttnParams p) {
   constexpr int DT = (HD16 + 1) / 2;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lr = lane & 31, lk = lane >> 5;
