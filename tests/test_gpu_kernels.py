@@ -339,6 +339,12 @@ ATT_CASES = [
     dict(nh=8, nkv=4, hd=64, bs=16, reqs=[(37, 128), (0, 100)], window=0, cap=50.0),
     dict(nh=4, nkv=2, hd=32, bs=16, reqs=[(11, 64), (70, 50)], window=40, cap=0.0),
     dict(nh=2, nkv=1, hd=128, bs=16, reqs=[(5, 256)], window=0, cap=30.0),
+    # decoded tokens whose window is much shorter than the context the step allows: the grid
+    # covers a window's blocks and counts them from the one each request's window begins in;
+    # the far key that stands out is the window's first, at, before and after a block's edge
+    dict(nh=8, nkv=4, hd=64, bs=16, reqs=[(254, 1), (255, 1), (298, 1), (299, 1), (554, 1), (555, 1), (810, 1),
+                                          (811, 1), (1499, 1), (39, 1)], window=300, cap=50.0),
+    dict(nh=4, nkv=2, hd=256, bs=16, reqs=[(1100, 1), (767, 1), (768, 1), (5, 1)], window=513, cap=0.0),
 ]
 
 

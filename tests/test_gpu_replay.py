@@ -266,6 +266,39 @@ def test_a_decoded_tokens_bits_do_not_depend_on_the_batch_in_bfloat16(tmp_path):
     assert np.abs(z[0] - alone_graph[0]).max() < 0.02 * np.abs(alone_graph[0]).max()
 
 
+def test_graphs_follow_a_context_across_the_lengths_they_cover(tmp_path):
+    """A bucket has a graph for each context length it has met, in steps of 1,024 tokens here.
+    A request that decodes from 1,019 to 1,030 tokens goes from the graph that covers 1,024 to
+    the one that covers 2,048 and gets the bits of eager steps all the way; so does a short
+    request beside it, whose windowed layers count their blocks from where its window begins."""
+    from zse_amd.engine.runner import StepEntry
+    from zse_amd.weights import write_random_model
+    cfg = dict(architectures=["Gemma2ForCausalLM"], model_type="gemma2", num_hidden_layers=2, hidden_size=64,
+               num_attention_heads=4, num_key_value_heads=2, head_dim=32, query_pre_attn_scalar=32,
+               intermediate_size=96, vocab_size=300, rope_theta=10000.0, sliding_window=200,
+               attn_logit_softcapping=30.0, final_logit_softcapping=20.0, rms_norm_eps=1e-6,
+               max_position_embeddings=4096)
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=6, std=0.08, gain_std=0.1, dtype="bfloat16",
+                                std_of={"embed_tokens": 0.02})
+    rng = np.random.default_rng(2)
+    streams = {"long": rng.integers(0, 300, 1018 + 12).tolist(), "short": rng.integers(0, 300, 290 + 12).tolist()}
+
+    def run(use_graphs):
+        runner = make_runner(folder, "bfloat16", page_size=16, cache_tokens=2048, max_seqs=2,
+                             max_batch_tokens=1024, max_model_len=4096, use_graphs=use_graphs)
+        for r, t in streams.items():
+            runner.step([StepEntry(r, t[:len(t) - 12], [])])
+        rows = []
+        for i in range(12):
+            rows.append(runner.step([StepEntry(r, [t[len(t) - 12 + i]], [0]) for r, t in streams.items()]).copy())
+        if use_graphs:
+            assert {k for k, g in runner.graphs.items() if isinstance(g, int)} == {(2, 1024), (2, 2048)}
+        runner.close()
+        return np.stack(rows)
+
+    assert np.array_equal(run(True), run(False))
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_steps_launched_from_their_written_down_lists(cases, dtype):
     """An eager step whose shape was seen before is launched by the native side from the list

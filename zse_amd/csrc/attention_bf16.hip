@@ -61,6 +61,7 @@ struct AttnParams {
   int tpw;                // tokens a wave owns
   int r_begin;            // first request of this launch
   int nchunks;            // split: chunks the grid covers
+  int from_window;        // decode: block 0 of a request is the one its window begins in
   int chunk;              // decoded tokens on 16-wide tiles: keys a wave takes, 32 or 64
 };
 
@@ -395,7 +396,11 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const int col = lane & 15, kq = lane >> 4;
   const int r = p.r_begin + blockIdx.z;
   const int kvh = blockIdx.y;
-  const int chunk = blockIdx.x * 4 + wave;
+  // Where the window is much shorter than the longest context, the grid covers a window's
+  // blocks only and counts them from the block the request's window begins in.
+  int block_x = blockIdx.x;
+  if (p.from_window) block_x += max(0, p.ctx_len[r] - p.window) / (4 * p.chunk);
+  const int chunk = block_x * 4 + wave;
   const int* table = p.block_table + (size_t)r * p.max_blocks;
   const int hd = p.hd, bsh = p.bs_shift, bmask = p.bs - 1, nkv = p.nkv;
   // The pages of the chunk's (up to two) tiles are asked for before the request's length is
@@ -415,6 +420,10 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   if (n <= 0) return;
   const int pos = p.ctx_len[r] - 1;
   const int row_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  // a block whose four chunks all lie past the context or before the window ends here, all
+  // its waves alike: the grid is sized for the longest context the caller allows
+  const int first_chunk = block_x * 4;
+  if (first_chunk * p.chunk > pos || first_chunk * p.chunk + 4 * p.chunk - 1 < row_lo) return;
   const int key_lo = max(row_lo, chunk * p.chunk);
   const int key_hi = min(pos, chunk * p.chunk + p.chunk - 1);
   const bool active = key_lo <= key_hi;          // a wave without keys still meets the others at the barrier
@@ -530,8 +539,6 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
     for (int dt = 0; dt < DT; dt++) *(f32x4*)(so + dt * 16 + 4 * kq) = o[dt];
   }
   __syncthreads();
-  const int first_chunk = blockIdx.x * 4;
-  if (first_chunk * p.chunk > pos || first_chunk * p.chunk + 4 * p.chunk - 1 < row_lo) return;
   for (int idx = threadIdx.x; idx < g * hd; idx += 256) {
     const int c = idx / hd, d = idx - c * hd;
     float mw[4], m = -INFINITY;
@@ -547,7 +554,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
       acc += e * sm_o[((size_t)w * g + c) * hd + d];
       l += e * sm_ml[(w * 16 + c) * 2 + 1];
     }
-    const size_t slot = ((size_t)(r - p.r_begin) * p.nh + kvh * g + c) * p.nchunks + blockIdx.x;
+    const size_t slot = ((size_t)(r - p.r_begin) * p.nh + kvh * g + c) * p.nchunks + block_x;
     p.part_o[slot * hd + d] = acc;
     if (d == 0) {
       p.part_ml[slot * 2] = m;
@@ -707,6 +714,7 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
   p.q_start = q_start; p.ctx_len = ctx_len; p.out = (__bf16*)out;
   p.nh = nh; p.nkv = nkv; p.hd = hd; p.bs = bs;
   p.scale = scale; p.softcap = softcap; p.window = window;
+  p.from_window = 0;
   p.bs_shift = 0;
   while ((1 << p.bs_shift) < bs) p.bs_shift++;
   const float log2e = 1.4426950408889634f;
@@ -743,6 +751,12 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
       // the block joins its four chunks: one partial result per 4 chunks of keys
       span = 4 * p.chunk;
       p.nchunks = grid.x;
+      // a window covers at most ceil(window / span) + 1 blocks of span keys
+      const int window_blocks = window > 0 ? (window + span - 1) / span + 1 : 0;
+      if (window > 0 && window_blocks < (int)grid.x) {
+        p.from_window = 1;
+        grid.x = window_blocks;
+      }
       p.part_ml = (float*)workspace + (size_t)n_dec * nh * p.nchunks * hd;
       const size_t lds = (4 * 16 * 2 + (size_t)4 * g * hd) * sizeof(float);
       switch (hd / 32) {

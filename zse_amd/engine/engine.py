@@ -293,6 +293,8 @@ class Engine:
         return self._stats
 
     def close(self) -> None:
+        if self.runner is not None:
+            self.runner.close()
         self.runner = None
         self.sampler = None
 

@@ -217,7 +217,7 @@ class StepRunner:
         self.meta_copied = rt.event()
         rt.record(self.meta_copied)
         self.logits: Optional[Tensor] = None
-        self.graphs: Dict[int, object] = {}      # bucket -> "warm" | graph handle
+        self.graphs: Dict[object, object] = {}   # bucket -> "warm"; (bucket, context covered) -> graph handle
         # a captured step replays the same launches with the same arguments: every part must
         # take what changes from step to step (tokens, positions, tables, slots) from device
         # memory alone.  The built-in parts do; a part says so with ``graph_safe = True``.
@@ -364,13 +364,21 @@ class StepRunner:
         return b if b <= self.max_seqs else 0
 
     def _graph_step(self, entries, bucket: int, tokens_from=None):
-        """One token for each request through the graph of this bucket.  The first step of
-        a bucket runs eagerly (it sizes the arena), the second is captured, later ones
-        replay.  Kernel arguments are fixed by the bucket: rows beyond the batch are
-        padding (position -1, no cache slot, no request), attention covers the longest
-        context the runner allows, and the logits land in a buffer of the graphs' own."""
+        """One token for each request through a graph of this bucket.  The first step of
+        a bucket runs eagerly (it sizes the arena), later ones are captured and replayed.
+        Kernel arguments are fixed by the graph: rows beyond the batch are padding (position
+        -1, no cache slot, no request), the logits land in a buffer of the graphs' own, and
+        attention covers a context length that is a step of an eighth of the longest the runner
+        allows (of 1,024 tokens at least), the first that holds the step's longest request: a
+        bucket has a graph for each such length it has met.  (The length only sizes the
+        attention kernels' grids; a block past a request's keys ends at once, but a grid of
+        mostly such blocks still costs time.)"""
         R = len(entries)
-        off, words, T, _, n_rows, host_entries, _, _, _ = self._pack(entries, bucket, bucket)
+        off, words, T, _, n_rows, host_entries, _, longest, _ = self._pack(entries, bucket, bucket)
+        grain = 1024
+        while grain * 8 < self.max_model_len:
+            grain *= 2
+        covered = min(-(-longest // grain) * grain, max(self.max_model_len, longest))
         logit_rows = self.meta_host.array(off["logit_rows"] * 4, bucket, np.int32)
         logit_rows[n_rows:] = 0
         self.rt.copy_h2d_async(self.meta_dev.ptr, self.meta_host.ptr, words * 4)
@@ -380,13 +388,13 @@ class StepRunner:
         if self.graph_logits is None:
             self.graph_logits = self.rt.empty((self.max_seqs, self.vocab), F32)
         out = self.graph_logits.rows(0, bucket)
-        state = self.graphs.get(bucket)
-        if isinstance(state, int):
-            self.rt.graph_launch(state)
+        graph = self.graphs.get((bucket, covered))
+        if graph is not None:
+            self.rt.graph_launch(graph)
             return self.graph_logits.rows(0, n_rows)
-        ctx = self._context(off, bucket, bucket, host_entries, 1, self.max_model_len, 0)
+        ctx = self._context(off, bucket, bucket, host_entries, 1, covered, 0)
         self.arena.reset()
-        if state is None:                       # first time: eager, lets the arena grow
+        if bucket not in self.graphs:           # first time: eager, lets the arena grow
             self.model.forward(ctx, self.caches, ctx.logit_rows, bucket, out)
             self.graphs[bucket] = "warm"
             return self.graph_logits.rows(0, n_rows)
@@ -399,9 +407,21 @@ class StepRunner:
                 graph = self.rt.capture_end()
         finally:
             self.arena.frozen = False
-        self.graphs[bucket] = graph
+        self.graphs[(bucket, covered)] = graph
         self.rt.graph_launch(graph)
         return self.graph_logits.rows(0, n_rows)
+
+    def close(self) -> None:
+        """Gives back what lives outside the runtime's memory pools: the captured graphs and
+        the launch lists.  The runner takes no step after this."""
+        self.rt.sync()
+        for key, g in list(self.graphs.items()):
+            if isinstance(g, int):
+                self.rt.graph_destroy(g)
+        self.graphs.clear()
+        for h in self.steplists.values():
+            self.k.steplist_destroy(h)
+        self.steplists.clear()
 
     MAX_STEPLISTS = 256
 
