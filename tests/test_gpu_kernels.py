@@ -550,7 +550,8 @@ def test_embed(rt, dtype, T, H, V):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("T,H,eps,uo", [(4, 96, 1e-5, 1), (3, 2304, 1e-6, 1), (2, 70, 1e-6, 0), (2, 9000, 1e-6, 1)])
+@pytest.mark.parametrize("T,H,eps,uo", [(4, 96, 1e-5, 1), (3, 2304, 1e-6, 1), (2, 70, 1e-6, 0), (2, 9000, 1e-6, 1),
+                                        (3, 3584, 1e-6, 1), (2, 4608, 1e-6, 1), (2, 7000, 1e-6, 0)])
 def test_rmsnorm_and_the_fused_joins(rt, dtype, T, H, eps, uo):
     k = rt.kernels(dtype)
     rng = np.random.default_rng(H)
@@ -591,14 +592,18 @@ def test_rmsnorm_and_the_fused_joins(rt, dtype, T, H, eps, uo):
     Hd2 = rt.upload(h)
     k.zk_norm_add_norm(ptr(up(rt, sub, dtype)), 0, None, 0.0, 0, Hd2.ptr, None, 0.0, 0, None, T, H, rt.stream)
     assert np.abs(rt.download(Hd2) - (h.astype(np.float64) + sub)).max() < 1e-6
-    # the sublayer's output as three planes of partial sums: the same bits as their sum, rounded
-    # to the activation type, gives when handed over as one tensor
-    planes = rng.normal(size=(3, T, H)).astype(np.float32)
-    total = (planes[0] + planes[1]) + planes[2]
+    # the sublayer's output as planes of partial sums (three; six for the wide rows, whose kernel
+    # takes them four a turn): the same bits as their sum in plane order, rounded to the
+    # activation type, gives when handed over as one tensor
+    P = 3 if H < 3000 else 6
+    planes = rng.normal(size=(P, T, H)).astype(np.float32)
+    total = planes[0]
+    for q in range(1, P):
+        total = total + planes[q]
     if dtype == "bfloat16":
         total = bf16(total)
     got = []
-    for src, parts in ((up(rt, total, dtype), 0), (rt.upload(planes), 3)):
+    for src, parts in ((up(rt, total, dtype), 0), (rt.upload(planes), P)):
         Hd3, nxt3 = rt.upload(h), rt.empty((T, H), dtype)
         k.zk_norm_add_norm(src.ptr, parts, W.ptr, eps, uo, Hd3.ptr, W2.ptr, eps * 2, uo, nxt3.ptr, T, H, rt.stream)
         got.append((rt.download(Hd3), rt.download_f32(nxt3)))

@@ -199,33 +199,83 @@ __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
   // every load is issued before the first sum is needed: one trip to memory, not three
   float v[MAXV][4], hv[MAXV][4], gp[MAXV][4], gn[MAXV][4];
   float ss = 0.f;
+  if constexpr (MAXV <= 3) {
+    // narrow rows: a vector's planes are summed where it is loaded (fewer registers; measured
+    // faster than the arrangement below at 2,304 columns)
 #pragma unroll
-  for (int j = 0; j < MAXV; j++) {
-    const int i = threadIdx.x * 4 + j * 1024;
-    if (i < H) {
-      if (parts <= 0) {
-        load4<act_t>(s + i, v[j]);
-      } else {
-        load4<float>(sf + i, v[j]);
-        // four planes a turn, their loads issued together; a plane past the last is read from
-        // the last and not added
-        for (int p0 = 1; p0 < parts; p0 += 4) {
-          float t[4][4];
+    for (int j = 0; j < MAXV; j++) {
+      const int i = threadIdx.x * 4 + j * 1024;
+      if (i < H) {
+        if (parts <= 0) {
+          load4<act_t>(s + i, v[j]);
+        } else {
+          load4<float>(sf + i, v[j]);
+          // four planes a turn, their loads issued together; a plane past the last is read from
+          // the last and not added
+          for (int p0 = 1; p0 < parts; p0 += 4) {
+            float t[4][4];
 #pragma unroll
-          for (int q = 0; q < 4; q++) load4<float>(sf + (size_t)min(p0 + q, parts - 1) * plane + i, t[q]);
+            for (int q = 0; q < 4; q++) load4<float>(sf + (size_t)min(p0 + q, parts - 1) * plane + i, t[q]);
 #pragma unroll
-          for (int q = 0; q < 4; q++)
-            if (p0 + q < parts) {
+            for (int q = 0; q < 4; q++)
+              if (p0 + q < parts) {
 #pragma unroll
-              for (int e = 0; e < 4; e++) v[j][e] += t[q][e];
-            }
+                for (int e = 0; e < 4; e++) v[j][e] += t[q][e];
+              }
+          }
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[j][e] = to_f32(from_f32<act_t>(v[j][e]));
+        }
+        load4<float>(hr + i, hv[j]);
+        if (w_post) load4<float>(w_post + i, gp[j]);
+        if (w_next) load4<float>(w_next + i, gn[j]);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < MAXV; j++) {
+      const int i = threadIdx.x * 4 + j * 1024;
+      if (i < H) {
+        if (parts <= 0) load4<act_t>(s + i, v[j]);
+        else load4<float>(sf + i, v[j]);
+        load4<float>(hr + i, hv[j]);
+        if (w_post) load4<float>(w_post + i, gp[j]);
+        if (w_next) load4<float>(w_next + i, gn[j]);
+      }
+    }
+    if (parts > 0) {
+      // wide rows: four planes a turn, the loads of the thread's whole share of the row issued
+      // together, so that a turn is one trip to memory whatever the width.  A plane past the
+      // last is read from the last and not added; the planes are added in their order.
+      for (int p0 = 1; p0 < parts; p0 += 4) {
+        float t[MAXV][4][4];
+#pragma unroll
+        for (int j = 0; j < MAXV; j++) {
+          const int i = threadIdx.x * 4 + j * 1024;
+          if (i < H) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) load4<float>(sf + (size_t)min(p0 + q, parts - 1) * plane + i, t[j][q]);
+          }
         }
 #pragma unroll
-        for (int e = 0; e < 4; e++) v[j][e] = to_f32(from_f32<act_t>(v[j][e]));
+        for (int j = 0; j < MAXV; j++) {
+          const int i = threadIdx.x * 4 + j * 1024;
+          if (i < H) {
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+              if (p0 + q < parts) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[j][e] += t[j][q][e];
+              }
+          }
+        }
       }
-      load4<float>(hr + i, hv[j]);
-      if (w_post) load4<float>(w_post + i, gp[j]);
-      if (w_next) load4<float>(w_next + i, gn[j]);
+#pragma unroll
+      for (int j = 0; j < MAXV; j++)
+        if (threadIdx.x * 4 + j * 1024 < H) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[j][e] = to_f32(from_f32<act_t>(v[j][e]));
+        }
     }
   }
 #pragma unroll
@@ -584,13 +634,17 @@ int zk_norm_add_norm(const void* sub, int sub_parts, const float* w_post, float 
   ZK_REQUIRE(w_next == nullptr || out != nullptr, "zk_norm_add_norm: next norm without output");
   if (T == 0) return 0;
   if (H % 4 == 0 && H <= NF_MAXV * 1024) {
-    if (H <= 3 * 1024)
-      norm_add_norm_fast_kernel<3><<<T, 256, 0, (hipStream_t)stream>>>(sub, sub_parts, w_post, eps_post, uo_post, h,
-                                                                       w_next, eps_next, uo_next, (act_t*)out, H);
-    else
-      norm_add_norm_fast_kernel<NF_MAXV><<<T, 256, 0, (hipStream_t)stream>>>(sub, sub_parts, w_post, eps_post,
-                                                                             uo_post, h, w_next, eps_next, uo_next,
-                                                                             (act_t*)out, H);
+    hipStream_t st = (hipStream_t)stream;
+#define ZK_NAN_(V)                                                                                              \
+  norm_add_norm_fast_kernel<V><<<T, 256, 0, st>>>(sub, sub_parts, w_post, eps_post, uo_post, h, w_next, eps_next, \
+                                                  uo_next, (act_t*)out, H)
+    // a thread holds ceil(H / 1024) vectors of four: the narrowest kernel that covers the row
+    const int vecs = (H + 1023) / 1024;
+    if (vecs <= 3) ZK_NAN_(3);
+    else if (vecs == 4) ZK_NAN_(4);
+    else if (vecs == 5) ZK_NAN_(5);
+    else ZK_NAN_(NF_MAXV);
+#undef ZK_NAN_
     return zk_launch_status("zk_norm_add_norm");
   }
   norm_add_norm_kernel<<<T, 256, 0, (hipStream_t)stream>>>(sub, sub_parts, w_post, eps_post, uo_post, h, w_next,
