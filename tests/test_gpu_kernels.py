@@ -345,6 +345,16 @@ ATT_CASES = [
     dict(nh=8, nkv=4, hd=64, bs=16, reqs=[(254, 1), (255, 1), (298, 1), (299, 1), (554, 1), (555, 1), (810, 1),
                                           (811, 1), (1499, 1), (39, 1)], window=300, cap=50.0),
     dict(nh=4, nkv=2, hd=256, bs=16, reqs=[(1100, 1), (767, 1), (768, 1), (5, 1)], window=513, cap=0.0),
+    # long portions (tiles shared by the groups of a block): a portion that starts inside a page
+    # and ends inside a tile, a window that begins inside a tile, pages of 8, 16, 32 and 64 keys,
+    # one, two, three and eight heads a KV head, a second request of another length in the launch
+    dict(nh=8, nkv=4, hd=256, bs=16, reqs=[(37, 300), (5, 70)], window=0, cap=50.0),
+    dict(nh=8, nkv=4, hd=128, bs=8, reqs=[(100, 333)], window=150, cap=30.0),
+    dict(nh=6, nkv=2, hd=64, bs=32, reqs=[(3, 260), (200, 45)], window=0, cap=0.0),
+    dict(nh=3, nkv=3, hd=32, bs=64, reqs=[(60, 500)], window=97, cap=20.0),
+    dict(nh=16, nkv=2, hd=16, bs=16, reqs=[(11, 190)], window=0, cap=50.0),
+    # so many groups (66 of 32 rows x 16 KV heads) that the choice by size takes the shared tiles
+    dict(nh=16, nkv=16, hd=16, bs=16, reqs=[(20, 2100)], window=700, cap=20.0),
 ]
 
 
@@ -406,22 +416,31 @@ def test_attention_over_pages(rt, kernel, case):
     QS, CL = rt.upload(qs), rt.upload(np.array(total, np.int32))
     tol = 2e-5 if dtype == "float32" else 0.02
     outs = []
-    for chunk in ((64, 32) if kernel == "mfma" else (0,)):      # both cuts of the decoded tokens' keys
+    # both cuts of the decoded tokens' keys; and every kernel for the portions: a group of rows a
+    # block (1), tiles shared by 4 or 8 groups (pages of 8 keys or more), the choice by size (0)
+    turns = [(0, 0)]
+    if kernel == "mfma":
+        turns = [(64, 0), (32, 0), (64, 1)] + ([(64, 4), (32, 8)] if bs >= 8 else [])
+    for chunk, portion_kernel in turns:
         OUT = rt.zeros((T, nh * hd), dtype)
         if kernel == "mfma":
+            k.zk_attention_bf16_portion_kernel(portion_kernel)
             n_multi = sum(1 for _, n in reqs if n > 1)
             # more context allowed than any request has, as in a captured step: more chunks than keys
             max_ctx = max(total) + 200
             ws = rt.zeros((max(1, k.zk_attention_bf16_workspace(R, nh, hd, max_ctx) // 4),), "float32")
-            k.zk_attention_bf16(Q.ptr, nh * hd, KC.ptr, VC.ptr, TBL.ptr, max_blocks, QS.ptr, CL.ptr, OUT.ptr,
-                                R, n_multi, max(n for _, n in reqs), max_ctx, nh, nkv, hd, bs, scale,
-                                c["cap"], c["window"], chunk, ws.ptr, ws.nbytes, rt.stream)
+            try:
+                k.zk_attention_bf16(Q.ptr, nh * hd, KC.ptr, VC.ptr, TBL.ptr, max_blocks, QS.ptr, CL.ptr, OUT.ptr,
+                                    R, n_multi, max(n for _, n in reqs), max_ctx, nh, nkv, hd, bs, scale,
+                                    c["cap"], c["window"], chunk, ws.ptr, ws.nbytes, rt.stream)
+            finally:
+                k.zk_attention_bf16_portion_kernel(0)
         else:
             k.zk_attention_plain(Q.ptr, nh * hd, KC.ptr, VC.ptr, TBL.ptr, max_blocks, REQ.ptr, POS.ptr, OUT.ptr,
                                  T, nh, nkv, hd, bs, scale, c["cap"], c["window"], 1 if vt else 0, rt.stream)
         got = rt.download_f32(OUT).reshape(T, nh, hd)
         err = np.abs(got - want)
-        assert err.max() < tol, (f"chunk {chunk}: max error {err.max()} at token "
+        assert err.max() < tol, (f"chunk {chunk}, portion kernel {portion_kernel}: max error {err.max()} at token "
                                  f"{np.unravel_index(err.argmax(), err.shape)}")
         outs.append(got)
 

@@ -385,6 +385,255 @@ __global__ __launch_bounds__(256, (HD16 <= 8 && !PAIR) ? 2 : 1) void attn_mfma_k
   }
 }
 
+// Long portions.  A block of NW waves owns NW groups of rows that follow each other in one
+// request (NW * tpw tokens times the g heads of a KV head), every wave one group, and all of
+// them walk the same keys: a tile of 32 keys and its values come from the cache once a block,
+// wait in LDS and serve every wave (attn_mfma_kernel fetches them once a group of 32 rows:
+// with many groups the way from L2 to the CUs then sets the time).  No join: a wave sees all
+// the keys of its rows.  Two buffers: the loads of the next tile are in flight while the
+// current one is multiplied, and one barrier a tile suffices.
+//   sK [2][32 keys][hd + 8]       a lane's piece for the first product is 16 bytes of a key's row
+//   sV [2][hd][32 + 8]            a channel's 32 keys in the order the second product wants:
+//                                 piece 2h + lk = keys 16h + 4lk + (0..3), 16h + 8 + 4lk + (0..3)
+// The padding of 16 bytes a row keeps the 16-byte reads of 16 lanes on different banks.
+// Pages of at least 8 keys (a 16-byte piece of the transposed V holds 8 keys of one page).
+template <int HD16, int NW>
+__global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_shared_kernel(AttnParams p) {
+  constexpr int HD = HD16 * 16, DT = (HD16 + 1) / 2;
+  constexpr int KLD = HD + 8, VLD = 32 + 8;
+  constexpr int NT = NW * 64;
+  constexpr int PIECES = 4 * HD;                        // 16-byte pieces of a K tile, and of a V tile
+  constexpr int PPT = (PIECES + NT - 1) / NT;           // pieces of each a thread moves
+  constexpr int CPK = HD / 8;                           // pieces of a key's row
+  extern __shared__ __attribute__((aligned(16))) unsigned char shared_raw[];
+  __bf16* sK = (__bf16*)shared_raw;                     // [2][32][KLD]
+  __bf16* sV = sK + 2 * 32 * KLD;                       // [2][HD][VLD]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 31, lk = lane >> 5;
+  const int r = p.r_begin + blockIdx.z;
+  int block_x, kvh;
+  portion_block(block_x, kvh);
+  const int qs = p.q_start[r], n = p.q_start[r + 1] - qs;
+  if (n <= 0) return;
+  const int start = p.ctx_len[r] - n;
+  const int per_block = NW * p.tpw;
+  // the last rows of a portion see the most keys and go first
+  const int bi = (n + per_block - 1) / per_block - 1 - block_x;
+  if (bi < 0) return;
+  const int g = p.nh / p.nkv;
+  // the block's keys: from the window of its first row to its last row
+  const int blk_lo = start + bi * per_block, blk_hi = start + min(n, (bi + 1) * per_block) - 1;
+  const int key_lo = p.window > 0 ? max(0, blk_lo - p.window + 1) : 0;
+  const int key_hi = blk_hi;
+  // the wave's rows
+  const int t0 = bi * per_block + wave * p.tpw;
+  const int ntok = max(0, min(p.tpw, n - t0));
+  const int tok = lr / g, hq = lr - tok * g;
+  const bool row_ok = tok < ntok;
+  const int trow = qs + (row_ok ? t0 + tok : 0);
+  const int pos = start + (row_ok ? t0 + tok : 0);
+  const int head = kvh * g + (row_ok ? hq : 0);
+  const int pos_lo = start + t0, pos_hi = start + t0 + ntok - 1;          // ntok == 0: no keys at all
+  const int row_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int all_hi = ntok * g == 32 ? pos_lo : -1;
+  const int all_lo = p.window > 0 ? max(0, pos_hi - p.window + 1) : 0;
+  const int* table = p.block_table + (size_t)r * p.max_blocks;
+  const int bsh = p.bs_shift, bmask = p.bs - 1, nkv = p.nkv;
+
+  bf16x8 qf[HD16];
+  {
+    const __bf16* qr = p.q + (size_t)trow * p.q_stride + (size_t)head * HD + lk * 8;
+#pragma unroll
+    for (int ks = 0; ks < HD16; ks++) {
+      if (row_ok) qf[ks] = *(const bf16x8*)(qr + ks * 16);
+      else
+#pragma unroll
+        for (int e = 0; e < 8; e++) qf[ks][e] = (__bf16)0.f;
+    }
+  }
+  f32x16 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) o[dt][e] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // The thread's pieces of a tile.  K: piece q is 8 channels (q % CPK) of key q / CPK.  V: the
+  // pieces of a page's part of the tile lie one behind the other in the cache, channel by
+  // channel: with tk = min(page size, 32) keys of a page in the tile, piece q is the keys
+  // [8c, 8c + 8) of channel d in part q / (HD tk / 8), d = (q / (tk / 8)) % HD, c = q % (tk / 8).
+  const int tk_shift = min(bsh, 5);                     // log2 of a page's keys in a tile
+  const int cpp_shift = tk_shift - 3;                   // log2 of the pieces of a channel in a page's part
+  int k_key[PPT], k_col[PPT], v_d[PPT], v_key[PPT];
+#pragma unroll
+  for (int j = 0; j < PPT; j++) {
+    const int q = min(tid + j * NT, PIECES - 1);
+    k_key[j] = q / CPK;
+    k_col[j] = (q % CPK) * 8;
+    const int part = q / (HD << cpp_shift), rem = q - part * (HD << cpp_shift);
+    v_d[j] = rem >> cpp_shift;
+    v_key[j] = (part << tk_shift) + ((rem & ((1 << cpp_shift) - 1)) << 3);
+  }
+  struct Pages { int k[PPT], v[PPT]; };
+  struct Stage { bf16x8 k[PPT], v[PPT]; };
+  // a key past the block's last reads that one again (it is masked), a piece of V past it the
+  // piece the last key lies in: every address stays inside the request's pages
+  auto look_up = [&](int key0, Pages& pg) {
+#pragma unroll
+    for (int j = 0; j < PPT; j++) {
+      pg.k[j] = table[min(key0 + k_key[j], key_hi) >> bsh];
+      pg.v[j] = table[min(key0 + v_key[j], key_hi & ~7) >> bsh];
+    }
+  };
+  auto fetch = [&](int key0, const Pages& pg, Stage& st) {
+#pragma unroll
+    for (int j = 0; j < PPT; j++) {
+      const int kk = min(key0 + k_key[j], key_hi);
+      st.k[j] = *(const bf16x8*)(p.kcache + ((((size_t)max(pg.k[j], 0) * nkv + kvh) << bsh) + (kk & bmask)) * HD +
+                                 k_col[j]);
+      const int kv = min(key0 + v_key[j], key_hi & ~7);
+      st.v[j] = *(const bf16x8*)(p.vcache + ((((size_t)max(pg.v[j], 0) * nkv + kvh) * HD + v_d[j]) << bsh) +
+                                 (kv & bmask));
+    }
+  };
+  auto stash = [&](int buf, const Stage& st) {
+    __bf16* kb = sK + buf * 32 * KLD;
+    __bf16* vb = sV + buf * HD * VLD;
+#pragma unroll
+    for (int j = 0; j < PPT; j++) {
+      if (PIECES % NT == 0 || tid + j * NT < PIECES) {
+        *(bf16x8*)(kb + k_key[j] * KLD + k_col[j]) = st.k[j];
+        // keys 8c + (0..3) go to piece 2h of the channel, keys 8c + 4 + (0..3) to piece 2h + 1,
+        // both at slot 4 (c % 2), with h = c / 2
+        const int c = v_key[j] >> 3;
+        __bf16* vrow = vb + v_d[j] * VLD + (c >> 1) * 16 + (c & 1) * 4;
+        bf16x4 lo4, hi4;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          lo4[e] = st.v[j][e];
+          hi4[e] = st.v[j][4 + e];
+        }
+        *(bf16x4*)vrow = lo4;
+        *(bf16x4*)(vrow + 8) = hi4;
+      }
+    }
+  };
+  const bool capped = p.softcap > 0.f;
+  auto tile = [&](int buf, int key0) {
+    const __bf16* kb = sK + buf * 32 * KLD + lr * KLD + lk * 8;
+    const __bf16* vb = sV + buf * HD * VLD + lk * 8;
+    // ---- S^T = K Q^T
+    f32x16 s;
+#pragma unroll
+    for (int e = 0; e < 16; e++) s[e] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < HD16; ks++)
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(kb + ks * 16), qf[ks], s, 0, 0, 0);
+    // ---- scale, cap, mask, running softmax (one query row per lane)
+    float mt = -INFINITY;
+    if (capped) {
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        const float ex = __builtin_amdgcn_exp2f(p.k2 * s[e]);
+        s[e] = p.c2 * (1.f - 2.f * __builtin_amdgcn_rcpf(ex + 1.f));
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 16; e++) s[e] *= p.k1;
+    }
+    if (key0 < all_lo || key0 + 31 > all_hi) {
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int key = key0 + 8 * j + 4 * lk + i;
+          const bool ok = row_ok && key >= row_lo && key <= pos;
+          s[4 * j + i] = ok ? s[4 * j + i] : -INFINITY;
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 16; e++) mt = fmaxf(mt, s[e]);
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = mt > m_run + 8.f ? mt : m_run;      // the maximum is followed lazily
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const bool moved = m_new > m_run;
+    const float corr = moved ? __builtin_amdgcn_exp2f(m_run - m_use) : 1.f;
+    float rs = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      const float pe = __builtin_amdgcn_exp2f(s[e] - m_use);
+      s[e] = pe;
+      rs += pe;
+    }
+    rs += __shfl_xor(rs, 32, 64);
+    l_run = l_run * corr + rs;
+    m_run = m_new;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) pb[h][e] = (__bf16)s[8 * h + e];
+    // ---- O^T = corr O^T + V^T P^T
+    if (__builtin_expect(__any(moved), 0)) {
+      // in the accumulation registers, where the products keep them
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+          float t;
+          asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
+                       : "+a"(o[dt][e]), "=&v"(t)
+                       : "v"(corr));
+        }
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+      const __bf16* vr = vb + min(dt * 32 + lr, HD - 1) * VLD;
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)vr, pb[0], o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8*)(vr + 16), pb[1], o[dt], 0, 0, 0);
+    }
+  };
+
+  // Every wave takes every tile of the block, also the few near the diagonal (or before its
+  // window) that none of its rows sees: masked, such a tile adds nothing, and a loop without a
+  // branch around the products lets the compiler leave the accumulators where they are (with
+  // the branch it copied all of them to ordinary registers on every turn: 852 instead of 1,135 us
+  // at 16 heads of 256).  The turn after the last tile fetches that tile again and leaves it
+  // unused.
+  {
+    int key0 = (key_lo / 32) * 32;
+    Pages pg, pn;
+    Stage st;
+    look_up(key0, pg);
+    fetch(key0, pg, st);
+    look_up(key0 + 32, pn);
+    stash(0, st);
+    __syncthreads();
+    for (int buf = 0; key0 <= key_hi; key0 += 32, buf ^= 1) {
+      fetch(key0 + 32, pn, st);
+      look_up(key0 + 64, pn);
+      tile(buf, key0);
+      stash(buf ^ 1, st);
+      __syncthreads();
+    }
+  }
+  if (!row_ok) return;
+  const float inv = 1.f / l_run;
+  __bf16* orow = p.out + ((size_t)trow * p.nh + head) * HD;
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int d = dt * 32 + 8 * j + 4 * lk;
+      if (d < HD) {
+        bf16x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (__bf16)(o[dt][4 * j + i] * inv);
+        *(bf16x4*)(orow + d) = w;
+      }
+    }
+}
+
 // One wave per (request, KV head, chunk of 64 keys) for requests that bring one token.
 // Columns of every tile are the g query heads of the KV head (col = lane % 16), rows are
 // keys (first product) or channels (second product).
@@ -647,7 +896,46 @@ static int launch_attn(const AttnParams& p, dim3 grid, hipStream_t s) {
   return zk_launch_status("zk_attention_bf16");
 }
 
+template <int HD16, int NW>
+static int launch_shared_one(const AttnParams& p, dim3 grid, hipStream_t s) {
+  constexpr int HD = HD16 * 16;
+  constexpr size_t lds = ((size_t)2 * 32 * (HD + 8) + (size_t)2 * HD * (32 + 8)) * sizeof(__bf16);
+  static bool prepared = false;
+  if (!prepared) {
+    if (lds > 64 * 1024 && hipFuncSetAttribute((const void*)attn_shared_kernel<HD16, NW>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return zk_fail("zk_attention_bf16: the shared-tile kernel's LDS buffers were refused");
+    prepared = true;
+  }
+  attn_shared_kernel<HD16, NW><<<grid, NW * 64, lds, s>>>(p);
+  return zk_launch_status("zk_attention_bf16 (shared tiles)");
+}
+
+template <int NW>
+static int launch_shared(const AttnParams& p, dim3 grid, hipStream_t s) {
+  switch (p.hd / 16) {
+    case 1: return launch_shared_one<1, NW>(p, grid, s);
+    case 2: return launch_shared_one<2, NW>(p, grid, s);
+    case 4: return launch_shared_one<4, NW>(p, grid, s);
+    case 8: return launch_shared_one<8, NW>(p, grid, s);
+    case 16:
+      if constexpr (NW <= 4) return launch_shared_one<16, NW>(p, grid, s);
+      else return zk_fail("zk_attention_bf16: eight waves a block take head sizes up to 128");
+    default: return zk_fail("zk_attention_bf16: head_dim must be 16, 32, 64, 128 or 256");
+  }
+}
+
+// 0: the portion kernel is chosen by the sizes; 1: a group of rows a block; 4, 8: shared
+// tiles with that many waves a block.  For tests and measurements (process-wide).
+static int portion_kernel_mode = 0;
+
 extern "C" {
+
+int zk_attention_bf16_portion_kernel(int mode) {
+  const int before = portion_kernel_mode;
+  if (mode == 0 || mode == 1 || mode == 4 || mode == 8) portion_kernel_mode = mode;
+  return before;
+}
 
 // 1 if the matrix-core kernel takes these sizes, else 0 (the caller then uses the plain kernel).
 int zk_attention_bf16_supports(int nh, int nkv, int hd, int bs) {
@@ -729,7 +1017,23 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
     // one block each) where single groups would need a second round
     const long long single = (long long)groups * nkv * r_prefill, paired = (long long)((groups + 1) / 2) * nkv * r_prefill;
     int rc;
-    if (single > 256 && paired <= 256) rc = launch_attn<false, true>(p, dim3((groups + 1) / 2, nkv, r_prefill), s);
+    // Many groups: tiles shared by the four or eight groups of a block, where that still gives
+    // every CU a block (four) or two (eight; head sizes up to 128, whose registers let two
+    // waves share a SIMD).  Measured at 8 to 32 heads of 128 and 256 with 512 to 4,096 rows:
+    // with fewer groups than that the kernel of one group a block is faster (at 2,048 rows of 8
+    // heads of 256: 75 us against 147), with more the shared tiles are (8 portions of 512 rows
+    // behind 7,680 tokens, 32 heads of 128: 1,630 -> 915 us; 16 heads of 256: 1,560 -> 1,125).
+    int shared_waves = 0;
+    if (bs >= 8 && portion_kernel_mode != 1) {
+      if (portion_kernel_mode > 1) shared_waves = portion_kernel_mode;
+      else if (single >= 4096 && hd <= 128) shared_waves = 8;
+      else if (single >= 1024) shared_waves = 4;
+      if (shared_waves == 8 && hd > 128) shared_waves = 4;       // no room for two waves a SIMD
+    }
+    if (shared_waves) {
+      dim3 grid((groups + shared_waves - 1) / shared_waves, nkv, r_prefill);
+      rc = shared_waves == 4 ? launch_shared<4>(p, grid, s) : launch_shared<8>(p, grid, s);
+    } else if (single > 256 && paired <= 256) rc = launch_attn<false, true>(p, dim3((groups + 1) / 2, nkv, r_prefill), s);
     else rc = launch_attn<false, false>(p, dim3(groups, nkv, r_prefill), s);
     if (rc) return rc;
   }
