@@ -1019,15 +1019,16 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
     int rc;
     // Many groups: tiles shared by the four or eight groups of a block, where that still gives
     // every CU a block (four) or two (eight; head sizes up to 128, whose registers let two
-    // waves share a SIMD).  Measured at 8 to 32 heads of 128 and 256 with 512 to 4,096 rows:
-    // with fewer groups than that the kernel of one group a block is faster (at 2,048 rows of 8
-    // heads of 256: 75 us against 147), with more the shared tiles are (8 portions of 512 rows
-    // behind 7,680 tokens, 32 heads of 128: 1,630 -> 915 us; 16 heads of 256: 1,560 -> 1,125).
+    // waves share a SIMD).  Measured at 8 to 32 heads of 128 and 256 with 512 to 8,192 rows:
+    // with fewer than about 768 groups the kernel of one group a block is faster (2,048 rows of
+    // 8 heads of 256, 512 groups: 75 us against 111; 768 groups: a tie), with more the shared
+    // tiles are (8 portions of 512 rows behind 7,680 tokens, 32 heads of 128: 1,630 -> 780 us;
+    // 16 heads of 256: 1,560 -> 845 us; 8,192 rows of 8 heads of 256: 877 -> 463 us).
     int shared_waves = 0;
     if (bs >= 8 && portion_kernel_mode != 1) {
       if (portion_kernel_mode > 1) shared_waves = portion_kernel_mode;
       else if (single >= 4096 && hd <= 128) shared_waves = 8;
-      else if (single >= 1024) shared_waves = 4;
+      else if (single >= 768) shared_waves = 4;
       if (shared_waves == 8 && hd > 128) shared_waves = 4;       // no room for two waves a SIMD
     }
     if (shared_waves) {
