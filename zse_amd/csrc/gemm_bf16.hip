@@ -7,8 +7,8 @@
 //    16x16x32 MFMAs straight from global memory: a lane's 16-byte load is exactly its MFMA
 //    operand (row = lane % 16, eight k values at 8 * (lane / 16)), so no LDS staging is
 //    needed.  Partial sums of the waves meet in LDS.
-//  * mid (17 <= M <= 64, strip layout): four strips a block, the activations of a k chunk
-//    shared through LDS, K split over blocks when N alone gives too few of them.
+//  * mid (17 <= M <= 64, strip layout): four strips a block, two waves each, the activations
+//    of a k chunk shared through LDS, K split over blocks when N alone gives too few of them.
 //  * tile (M > 64, prefill): 256x256x64 (sixteen waves), 128x256x64 (eight) or 128x128x64 (four)
 //    block tiles staged through LDS, each wave a 64x64 corner built from 32x32x16 MFMAs.
 // Epilogues: plain store (bf16 or float), soft cap on float output (LM head), and
@@ -698,10 +698,10 @@ static bool joinable_by_reader(int N, int ldc, int c_is_f32, int epi) {
 // ------------------------------------------------------------------ mid (16 < M <= 64)
 // With more than one column tile the activations weigh more than the weights on the way
 // from L2 to the CUs when every 16-row strip fetches them again (64 rows of A per 16 rows
-// of W).  Here a block owns four strips, one per wave, all four walk K together, and the
+// of W).  Here a block owns four strips, a pair of waves each, all walk K together, and the
 // activations of the current 256-wide k chunk wait in LDS for all of them: 64 rows of A per
-// 64 rows of W.  Weights come straight from global memory in strip layout, the next chunk's
-// loads are in flight while the current one is multiplied.
+// 64 rows of W.  Weights come straight from global memory in strip layout, the loads of the
+// next two chunks are in flight while the current one is multiplied.
 //
 // Few column blocks (N of a few thousand) cannot fill 256 CUs, so blockIdx.y splits K into
 // `ksplit` ranges.  Then each block leaves its partial sums in the workspace and a second,
@@ -733,15 +733,26 @@ __device__ __forceinline__ void mid_store(const f32x4 (&acc)[GATED ? 2 : 1][MT],
   }
 }
 
+// Eight waves a block, two for each of its four strips: waves 0..3 take the first half of a
+// chunk's steps, waves 4..7 the second, and the second wave's sums reach the first through LDS
+// at the end.  A wave holds three chunks' weights in registers (one being multiplied, two on
+// their way) and the activations have three buffers in LDS: a chunk's products take less time
+// than a load (at 64 rows with a gate about 1.2 us against 2 us), so with one chunk on its way
+// every chunk waited for its loads, and where the column blocks are too few for a second block
+// on the CU (N = 9216 with a gate: 144 blocks) nothing filled the wait.  Against four waves with
+// one chunk ahead: 5 to 17 % less time at 24 to 64 rows on the layer shapes of the 2B, 9B and
+// 27B models (2B down at 64 rows 15.4 -> 13.1 us, 9B down at 32 rows 25.0 -> 21.2 us); two waves
+// a strip alone, without the second chunk ahead, gave 0 to 3 %.
 template <int MT, bool GATED>
-__global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict__ A, int lda,
-                                                       const __bf16* __restrict__ W,
-                                                       void* __restrict__ C, int ldc, int c_is_f32,
-                                                       int M, int N, int K, int epi, float cap,
-                                                       float* __restrict__ partials, int ksplit) {
+__global__ __launch_bounds__(512) void gemm_mid_kernel(const __bf16* __restrict__ A, int lda,
+                                                        const __bf16* __restrict__ W,
+                                                        void* __restrict__ C, int ldc, int c_is_f32,
+                                                        int M, int N, int K, int epi, float cap,
+                                                        float* __restrict__ partials, int ksplit) {
   constexpr int NS = GATED ? 2 : 1;
-  __shared__ __bf16 sA[2][MT * 16][GM_LD];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int WSTEPS = GM_STEPS / 2;                  // steps of a chunk a wave multiplies
+  __shared__ __bf16 sA[3][MT * 16][GM_LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3, khalf = tid >> 8;
   const int r = lane & 15, kq = lane >> 4;
   const int ksteps = K / 32;
   const int s_begin = (int)((long)blockIdx.y * ksteps / ksplit);
@@ -752,23 +763,22 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
   const __bf16* wp[NS];
   wp[0] = W + (size_t)(strip_ok ? strip : 0) * ksteps * 512 + lane * 8;
   if (GATED) wp[NS - 1] = W + ((size_t)(N / 16) + (strip_ok ? strip : 0)) * ksteps * 512 + lane * 8;
-  // A pieces of a chunk: MT*16 rows x 32 pieces of 16 bytes; a wave reads two rows' 512 contiguous bytes
-  constexpr int APT = MT * 16 * 32 / 256;
-  const int a_piece = tid & 31, a_row0 = tid >> 5;     // rows a_row0 + 8 j
+  // A pieces of a chunk: MT*16 rows x 32 pieces of 16 bytes, 16 rows a pass of the 512 threads
+  constexpr int APT = MT * 16 * 32 / 512;
+  const int a_piece = tid & 31, a_row0 = tid >> 5;
   f32x4 acc[NS][MT];
 #pragma unroll
   for (int g = 0; g < NS; g++)
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) acc[g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // Every load is issued, none under a condition (loads under a branch make the compiler wait
-  // for all loads in flight before the first use of any): a step past the range reads the
-  // range's last step again, a row past M row M - 1, and the activations are set to zero
-  // afterwards where they lie outside, which makes the product nothing whatever the weights.
+  // Every load is issued, none under a condition: a step past the range reads the range's last
+  // step again, a row past M row M - 1; activations outside are set to zero afterwards, which
+  // makes the product nothing whatever the weights.
   auto fetch_a = [&](int s0, bf16x8 (&ra)[APT]) {
 #pragma unroll
     for (int j = 0; j < APT; j++) {
-      const int row = a_row0 + 8 * j;
+      const int row = a_row0 + 16 * j;
       const bool in = row < M && s0 + a_piece / 4 < s_end;
       const int step = min(s0 + a_piece / 4, s_end - 1);
       const bf16x8 v = *(const bf16x8*)(A + (size_t)min(row, M - 1) * lda + step * 32 + (a_piece % 4) * 8);
@@ -777,52 +787,71 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const __bf16* __restrict_
   };
   auto stash_a = [&](int buf, const bf16x8 (&ra)[APT]) {
 #pragma unroll
-    for (int j = 0; j < APT; j++) *(bf16x8*)(&sA[buf][a_row0 + 8 * j][a_piece * 8]) = ra[j];
+    for (int j = 0; j < APT; j++) *(bf16x8*)(&sA[buf][a_row0 + 16 * j][a_piece * 8]) = ra[j];
   };
-  auto fetch_w = [&](int s0, bf16x8 (&wf)[NS][GM_STEPS]) {
+  auto fetch_w = [&](int s0, bf16x8 (&wf)[NS][WSTEPS]) {
 #pragma unroll
-    for (int s = 0; s < GM_STEPS; s++)
+    for (int s = 0; s < WSTEPS; s++)
 #pragma unroll
       for (int g = 0; g < NS; g++)
-        wf[g][s] = *(const bf16x8*)(wp[g] + (size_t)min(s0 + s, s_end - 1) * 512);
+        wf[g][s] = *(const bf16x8*)(wp[g] + (size_t)min(s0 + khalf * WSTEPS + s, s_end - 1) * 512);
   };
-  auto multiply = [&](int buf, const bf16x8 (&wf)[NS][GM_STEPS]) {
+  auto multiply = [&](int buf, const bf16x8 (&wf)[NS][WSTEPS]) {
 #pragma unroll
-    for (int s = 0; s < GM_STEPS; s++)
+    for (int s = 0; s < WSTEPS; s++)
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) {
-        const bf16x8 af = *(const bf16x8*)(&sA[buf][mt * 16 + r][s * 32 + kq * 8]);
+        const bf16x8 af = *(const bf16x8*)(&sA[buf][mt * 16 + r][(khalf * WSTEPS + s) * 32 + kq * 8]);
 #pragma unroll
         for (int g = 0; g < NS; g++)
           acc[g][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g][s], af, acc[g][mt], 0, 0, 0);
       }
   };
 
-  bf16x8 ra[APT], w0[NS][GM_STEPS], w1[NS][GM_STEPS];
-  fetch_a(s_begin, ra);
+  // Chunk c: its activations wait in LDS buffer c % 3, its weights in register set c % 3; the
+  // activations of chunk c + 1 are in register set (c + 1) % 2 on their way to LDS.  A turn
+  // asks for chunk c + 2, multiplies chunk c, puts chunk c + 1's activations into LDS.
+  bf16x8 ra0[APT], ra1[APT], w0[NS][WSTEPS], w1[NS][WSTEPS], w2[NS][WSTEPS];
+  fetch_a(s_begin, ra0);
   fetch_w(s_begin, w0);
-  stash_a(0, ra);
+  fetch_a(s_begin + GM_STEPS, ra1);
+  fetch_w(s_begin + GM_STEPS, w1);
+  stash_a(0, ra0);
   __syncthreads();
-  for (int s0 = s_begin; s0 < s_end; s0 += 2 * GM_STEPS) {
-    const bool more1 = s0 + GM_STEPS < s_end;
-    if (more1) {
-      fetch_a(s0 + GM_STEPS, ra);
-      fetch_w(s0 + GM_STEPS, w1);
-    }
-    multiply(0, w0);
-    if (!more1) break;
-    stash_a(1, ra);
-    __syncthreads();
-    const bool more2 = s0 + 2 * GM_STEPS < s_end;
-    if (more2) {
-      fetch_a(s0 + 2 * GM_STEPS, ra);
-      fetch_w(s0 + 2 * GM_STEPS, w0);
-    }
-    multiply(1, w1);
-    if (!more2) break;
-    stash_a(0, ra);
-    __syncthreads();
+#define ZK_MID8_TURN(BUF, WCUR, WNEXT2, RA_NEXT2, RA_NEXT1)   \
+  fetch_a(s0 + 2 * GM_STEPS, RA_NEXT2);                       \
+  fetch_w(s0 + 2 * GM_STEPS, WNEXT2);                         \
+  multiply(BUF, WCUR);                                        \
+  s0 += GM_STEPS;                                             \
+  if (s0 >= s_end) break;                                     \
+  stash_a((BUF + 1) % 3, RA_NEXT1);                           \
+  __syncthreads();
+  for (int s0 = s_begin;;) {
+    ZK_MID8_TURN(0, w0, w2, ra0, ra1)
+    ZK_MID8_TURN(1, w1, w0, ra1, ra0)
+    ZK_MID8_TURN(2, w2, w1, ra0, ra1)
+    ZK_MID8_TURN(0, w0, w2, ra1, ra0)
+    ZK_MID8_TURN(1, w1, w0, ra0, ra1)
+    ZK_MID8_TURN(2, w2, w1, ra1, ra0)
   }
+#undef ZK_MID8_TURN
+  // the second wave of each strip hands its sums over (the activation buffers are free once
+  // every wave has left the loop); first half + second half, in that order
+  __syncthreads();
+  static_assert(sizeof(sA) >= (size_t)4 * NS * MT * 64 * sizeof(f32x4), "no room to hand the sums over");
+  f32x4* hand = (f32x4*)&sA[0][0][0] + ((size_t)wave * NS * MT) * 64 + lane;
+  if (khalf == 1) {
+#pragma unroll
+    for (int g = 0; g < NS; g++)
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) hand[(g * MT + mt) * 64] = acc[g][mt];
+  }
+  __syncthreads();
+  if (khalf == 1) return;
+#pragma unroll
+  for (int g = 0; g < NS; g++)
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) acc[g][mt] += hand[(g * MT + mt) * 64];
   if (ksplit > 1) {
     // the range's partial sums: plane (range, g) of [M, npad] floats
     if (!strip_ok) return;
@@ -869,6 +898,7 @@ __global__ __launch_bounds__(256) void gemm_join_kernel(const float* __restrict_
   }
 }
 
+
 template <bool GATED>
 static int launch_mid(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M, int N,
                       int K, int epi, float cap, const GemmWorkspace& wsp, int* parts, hipStream_t s) {
@@ -896,7 +926,7 @@ static int launch_mid(const void* A, int lda, const void* W, void* C, int ldc, i
   float* partials = (float*)ws;
   dim3 grid(cblocks, ksplit);
 #define ZK_MID(MT_)                                                                                   \
-  gemm_mid_kernel<MT_, GATED><<<grid, 256, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, \
+  gemm_mid_kernel<MT_, GATED><<<grid, 512, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, \
                                                    M, N, K, epi, cap, partials, ksplit)
   if (mt == 2) { ZK_MID(2); }
   else if (mt == 3) { ZK_MID(3); }
