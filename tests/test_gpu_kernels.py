@@ -122,7 +122,10 @@ def test_gemm_bf16_gated_epilogue(rt, M, I, K, act):
                                           (64, 320, 800, True), (40, 336, 256, True), (33, 48, 1056, True),
                                           # over 64 rows, few tiles, long K: k ranges over blocks, then a join
                                           (100, 200, 2048, False), (130, 336, 2048, True), (70, 90, 4128, False),
-                                          (512, 2304, 9216, False)])
+                                          (512, 2304, 9216, False),
+                                          # 17..64 rows, more than 512 strips: three strips a block
+                                          # (the last block not full, the last strip not whole)
+                                          (40, 8224, 288, True), (64, 9216, 2304, True), (24, 8200, 320, False)])
 def test_gemm_bf16_strip_layout(rt, M, N, K, gated):
     """The same products with the weights rearranged into strips of 16 rows by 32 columns, and
     an embedding gather out of that layout."""

@@ -748,7 +748,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const __bf16* __restrict_
                                                         const __bf16* __restrict__ W,
                                                         void* __restrict__ C, int ldc, int c_is_f32,
                                                         int M, int N, int K, int epi, float cap,
-                                                        float* __restrict__ partials, int ksplit) {
+                                                        float* __restrict__ partials, int ksplit, int spb) {
   constexpr int NS = GATED ? 2 : 1;
   constexpr int WSTEPS = GM_STEPS / 2;                  // steps of a chunk a wave multiplies
   __shared__ __bf16 sA[3][MT * 16][GM_LD];
@@ -758,11 +758,16 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const __bf16* __restrict_
   const int s_begin = (int)((long)blockIdx.y * ksteps / ksplit);
   const int s_end = (int)((long)(blockIdx.y + 1) * ksteps / ksplit);
   const int nstrips = (N + 15) / 16;
-  const int strip = blockIdx.x * 4 + wave;
-  const bool strip_ok = strip < nstrips;
+  // spb strips a block (3 where that spreads the strips more evenly over the CUs).  The waves of
+  // the fourth place then do the first place's work over again and store nothing: their loads
+  // hit what the first place's waves have just fetched, and a branch around loads would make
+  // the compiler wait for every load in flight.
+  const int strip = blockIdx.x * spb + (wave < spb ? wave : 0);
+  const bool strip_ok = wave < spb && strip < nstrips;
+  const int strip_read = strip < nstrips ? strip : 0;
   const __bf16* wp[NS];
-  wp[0] = W + (size_t)(strip_ok ? strip : 0) * ksteps * 512 + lane * 8;
-  if (GATED) wp[NS - 1] = W + ((size_t)(N / 16) + (strip_ok ? strip : 0)) * ksteps * 512 + lane * 8;
+  wp[0] = W + (size_t)strip_read * ksteps * 512 + lane * 8;
+  if (GATED) wp[NS - 1] = W + ((size_t)(N / 16) + strip_read) * ksteps * 512 + lane * 8;
   // A pieces of a chunk: MT*16 rows x 32 pieces of 16 bytes, 16 rows a pass of the 512 threads
   constexpr int APT = MT * 16 * 32 / 512;
   const int a_piece = tid & 31, a_row0 = tid >> 5;
@@ -904,7 +909,18 @@ static int launch_mid(const void* A, int lda, const void* W, void* C, int ldc, i
                       int K, int epi, float cap, const GemmWorkspace& wsp, int* parts, hipStream_t s) {
   const int mt = (M + 15) / 16;
   const int npad = (N + 15) / 16 * 16;
-  const int cblocks = ((N + 15) / 16 + 3) / 4;
+  const int nstrips = (N + 15) / 16;
+  // Strips a block: four, or three where the blocks of four fill the CUs unevenly and K is not
+  // split anyway (N = 9216 with a gate is 576 strips: 144 blocks of four leave 112 CUs idle, 192
+  // blocks of three give every busy CU a quarter less to read: 28.0 -> 24.6 us at 64 rows;
+  // 2304 strips: three rounds of blocks either way, 157 -> 146 us).  What counts is the most
+  // strips a CU gets, rounds of 256 blocks times the strips of a block.
+  int spb = 4;
+  {
+    auto most = [&](int b) { return (long)(((nstrips + b - 1) / b + 255) / 256) * b; };
+    if ((nstrips + 3) / 4 > 128 && most(3) * 10 <= most(4) * 9) spb = 3;
+  }
+  const int cblocks = (nstrips + spb - 1) / spb;
   // Split K until every CU has a block, a range no shorter than a chunk of GM_STEPS steps; two
   // blocks a CU where ranges stay long (16 chunks or more: the blocks of a CU then cover each
   // other's waits).  More ranges than that cost more in partial sums than they gain.  The
@@ -927,7 +943,7 @@ static int launch_mid(const void* A, int lda, const void* W, void* C, int ldc, i
   dim3 grid(cblocks, ksplit);
 #define ZK_MID(MT_)                                                                                   \
   gemm_mid_kernel<MT_, GATED><<<grid, 512, 0, s>>>((const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, \
-                                                   M, N, K, epi, cap, partials, ksplit)
+                                                   M, N, K, epi, cap, partials, ksplit, spb)
   if (mt == 2) { ZK_MID(2); }
   else if (mt == 3) { ZK_MID(3); }
   else { ZK_MID(4); }
