@@ -351,7 +351,7 @@ ATT_CASES = [
     # long portions (tiles shared by the groups of a block): a portion that starts inside a page
     # and ends inside a tile, a window that begins inside a tile, pages of 8, 16, 32 and 64 keys,
     # one, two, three and eight heads a KV head, a second request of another length in the launch
-    dict(nh=8, nkv=4, hd=256, bs=16, reqs=[(37, 300), (5, 70)], window=0, cap=50.0),
+    dict(nh=8, nkv=4, hd=256, bs=16, reqs=[(37, 300), (5, 70)], window=0, cap=50.0, ranges_by_size=True),
     dict(nh=8, nkv=4, hd=128, bs=8, reqs=[(100, 333)], window=150, cap=30.0),
     dict(nh=6, nkv=2, hd=64, bs=32, reqs=[(3, 260), (200, 45)], window=0, cap=0.0),
     dict(nh=3, nkv=3, hd=32, bs=64, reqs=[(60, 500)], window=97, cap=20.0),
@@ -420,10 +420,11 @@ def test_attention_over_pages(rt, kernel, case):
     tol = 2e-5 if dtype == "float32" else 0.02
     outs = []
     # both cuts of the decoded tokens' keys; and every kernel for the portions: a group of rows a
-    # block (1), tiles shared by 4 or 8 groups (pages of 8 keys or more), the choice by size (0)
+    # block (1), tiles shared by 4 or 8 groups (pages of 8 keys or more), shared tiles with the keys
+    # in ranges and a join (5; long contexts, else as 4), the choice by size (0)
     turns = [(0, 0)]
     if kernel == "mfma":
-        turns = [(64, 0), (32, 0), (64, 1)] + ([(64, 4), (32, 8)] if bs >= 8 else [])
+        turns = [(64, 0), (32, 0), (64, 1)] + ([(64, 4), (32, 8), (64, 5)] if bs >= 8 else [])
     for chunk, portion_kernel in turns:
         OUT = rt.zeros((T, nh * hd), dtype)
         if kernel == "mfma":
@@ -431,7 +432,9 @@ def test_attention_over_pages(rt, kernel, case):
             n_multi = sum(1 for _, n in reqs if n > 1)
             # more context allowed than any request has, as in a captured step: more chunks than keys
             max_ctx = max(total) + 200
-            ws = rt.zeros((max(1, k.zk_attention_bf16_workspace(R, nh, hd, max_ctx) // 4),), "float32")
+            ws_bytes = (k.zk_attention_bf16_workspace(R, nh, hd, max_ctx) + 255) // 256 * 256
+            ws_bytes += k.zk_attention_bf16_portion_workspace(max(1, n_multi) * (max(n for _, n in reqs) + 128), nh, nkv, hd)
+            ws = rt.zeros((ws_bytes // 4 + 1,), "float32")
             try:
                 k.zk_attention_bf16(Q.ptr, nh * hd, KC.ptr, VC.ptr, TBL.ptr, max_blocks, QS.ptr, CL.ptr, OUT.ptr,
                                     R, n_multi, max(n for _, n in reqs), max_ctx, nh, nkv, hd, bs, scale,
@@ -446,6 +449,9 @@ def test_attention_over_pages(rt, kernel, case):
         assert err.max() < tol, (f"chunk {chunk}, portion kernel {portion_kernel}: max error {err.max()} at token "
                                  f"{np.unravel_index(err.argmax(), err.shape)}")
         outs.append(got)
+    if kernel == "mfma" and c.get("ranges_by_size"):
+        # few blocks of rows, 17 tiles of keys: the choice by size cuts the keys into ranges
+        assert np.array_equal(outs[0], outs[turns.index((64, 5))]) and not np.array_equal(outs[0], outs[turns.index((64, 4))])
 
 
 def run_attention(rt, kernel, q, kk, vv, past, nh, nkv, hd, bs, scale, cap, window, chunk=64, max_ctx=None):

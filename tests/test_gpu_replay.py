@@ -299,6 +299,41 @@ def test_graphs_follow_a_context_across_the_lengths_they_cover(tmp_path):
     assert np.array_equal(run(True), run(False))
 
 
+def test_a_portion_behind_a_long_context_against_the_whole_prompt(tmp_path):
+    """A portion of 64 tokens behind 836 others (its attention cuts the keys into ranges that a
+    second kernel joins), then one of 40 behind 900 and decoded tokens, against the same prompt
+    fed whole and against the 32-bit path."""
+    from zse_amd.engine.runner import StepEntry
+    from zse_amd.weights import write_random_model
+    cfg = dict(architectures=["Gemma2ForCausalLM"], model_type="gemma2", num_hidden_layers=2, hidden_size=64,
+               num_attention_heads=4, num_key_value_heads=2, head_dim=32, query_pre_attn_scalar=32,
+               intermediate_size=96, vocab_size=300, rope_theta=10000.0, sliding_window=600,
+               attn_logit_softcapping=30.0, final_logit_softcapping=20.0, rms_norm_eps=1e-6,
+               max_position_embeddings=2048)
+    folder = write_random_model(str(tmp_path / "m"), cfg, seed=8, std=0.08, gain_std=0.1, dtype="bfloat16",
+                                std_of={"embed_tokens": 0.02})
+    rng = np.random.default_rng(3)
+    toks = rng.integers(0, 300, 944).tolist()
+
+    def run(dtype, cuts):
+        runner = make_runner(folder, dtype, page_size=16, cache_tokens=1024, max_seqs=2, max_batch_tokens=1024,
+                             max_model_len=1024)
+        at, rows = 0, []
+        for n in cuts:
+            z = runner.step([StepEntry("a", toks[at:at + n], [i for i in range(n) if at + i >= 836])])
+            rows += [row.copy() for row in z]
+            at += n
+        runner.close()
+        return np.stack(rows)
+
+    cut = run("bfloat16", [836, 64, 40, 1, 1, 1, 1])
+    whole = run("bfloat16", [940, 1, 1, 1, 1])
+    want = run("float32", [940, 1, 1, 1, 1])
+    assert cut.shape == whole.shape == want.shape == (108, 300)
+    assert_close(cut, want, "bfloat16", "portions behind a long context")
+    assert_close(whole, want, "bfloat16", "the whole prompt")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_steps_launched_from_their_written_down_lists(cases, dtype):
     """An eager step whose shape was seen before is launched by the native side from the list

@@ -29,6 +29,8 @@
 // halves both the accumulator registers and the wasted work, so two waves fit a SIMD.
 #include "common.h"
 
+#include <algorithm>
+
 #if ZSE_ACT_BF16
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -37,6 +39,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 #define ATT_CHUNK 64
+#define ATT_MOST_RANGES 8      // ranges of keys a block of rows of a portion is cut into, at most
 
 struct AttnParams {
   const __bf16* q;
@@ -397,7 +400,13 @@ __global__ __launch_bounds__(256, (HD16 <= 8 && !PAIR) ? 2 : 1) void attn_mfma_k
 //                                 piece 2h + lk = keys 16h + 4lk + (0..3), 16h + 8 + 4lk + (0..3)
 // The padding of 16 bytes a row keeps the 16-byte reads of 16 lanes on different banks.
 // Pages of at least 8 keys (a 16-byte piece of the transposed V holds 8 keys of one page).
-template <int HD16, int NW>
+//
+// SPLIT: a launch of few blocks with many keys each (a prompt of a few thousand tokens and few
+// heads) cuts the keys of a block of rows into ranges of p.chunk tiles, counted from the
+// block's first tile; blockIdx.x is (block of rows) * p.nchunks + range.  A block then leaves
+// (max, sum, O) of its range for every row, as the chunks of a decoded token do, and
+// attn_portion_join_kernel joins a row's ranges in their order.
+template <int HD16, int NW, bool SPLIT>
 __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_shared_kernel(AttnParams p) {
   constexpr int HD = HD16 * 16, DT = (HD16 + 1) / 2;
   constexpr int KLD = HD + 8, VLD = 32 + 8;
@@ -418,13 +427,21 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
   const int start = p.ctx_len[r] - n;
   const int per_block = NW * p.tpw;
   // the last rows of a portion see the most keys and go first
-  const int bi = (n + per_block - 1) / per_block - 1 - block_x;
+  const int rows_x = SPLIT ? block_x / p.nchunks : block_x;
+  const int range = SPLIT ? block_x - rows_x * p.nchunks : 0;
+  const int bi = (n + per_block - 1) / per_block - 1 - rows_x;
   if (bi < 0) return;
   const int g = p.nh / p.nkv;
   // the block's keys: from the window of its first row to its last row
   const int blk_lo = start + bi * per_block, blk_hi = start + min(n, (bi + 1) * per_block) - 1;
-  const int key_lo = p.window > 0 ? max(0, blk_lo - p.window + 1) : 0;
-  const int key_hi = blk_hi;
+  int key_lo = p.window > 0 ? max(0, blk_lo - p.window + 1) : 0;
+  int key_hi = blk_hi;
+  if (SPLIT) {
+    const int first_tile = key_lo / 32 + range * p.chunk;
+    if (first_tile * 32 > key_hi) return;              // the block of rows has fewer ranges
+    key_lo = max(key_lo, first_tile * 32);
+    key_hi = min(key_hi, (first_tile + p.chunk) * 32 - 1);
+  }
   // the wave's rows
   const int t0 = bi * per_block + wave * p.tpw;
   const int ntok = max(0, min(p.tpw, n - t0));
@@ -617,7 +634,22 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
       __syncthreads();
     }
   }
-  if (!row_ok) return;
+  if (!SPLIT && !row_ok) return;
+  if (SPLIT) {
+    // A wave's results of its range, as they lie in its registers: 16 bytes a lane, a wave's 64
+    // lanes one contiguous KB per (dt, j), so every store is whole lines (stored row by row, a
+    // lane's pieces are 32 bytes here and 32 there: measured three times slower).  The joining
+    // kernel reads them back with the same lanes.  Every lane stores, rows or not.
+    const size_t slot = ((((size_t)blockIdx.z * p.nkv + kvh) * (gridDim.x / p.nchunks) + rows_x) * p.nchunks + range) * NW + wave;
+    p.part_ml[slot * 128 + lane] = lk == 0 ? m_run : l_run;
+    f32x4* po = (f32x4*)p.part_o + slot * (DT * 4 * 64) + lane;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        po[(dt * 4 + j) * 64] = f32x4{o[dt][4 * j], o[dt][4 * j + 1], o[dt][4 * j + 2], o[dt][4 * j + 3]};
+    return;
+  }
   const float inv = 1.f / l_run;
   __bf16* orow = p.out + ((size_t)trow * p.nh + head) * HD;
 #pragma unroll
@@ -632,6 +664,59 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
         *(bf16x4*)(orow + d) = w;
       }
     }
+}
+
+// Joins the ranges of keys of a portion's rows (attn_shared_kernel, SPLIT), in their order: a
+// block of 64 threads per (32 channels of a wave of a block of rows, KV head, request), every
+// lane the row and the channels it had in the kernel that wrote the partial results.  The ranges a block of rows
+// has follow from its first and last key as there; a range that a row does not see at all (one
+// past its position, in a block of rows on the diagonal) has the maximum -inf and weighs nothing.
+__global__ __launch_bounds__(64) void attn_portion_join_kernel(AttnParams p, int per_block, int row_blocks, int dts) {
+  const int r = p.r_begin + blockIdx.z, kvh = blockIdx.y;
+  const int dt = blockIdx.x % dts, ww = blockIdx.x / dts;      // 32 channels of a wave's rows a block
+  const int rows_x = ww >> 2, wave = ww & 3;
+  const int lane = threadIdx.x, lr = lane & 31, lk = lane >> 5;
+  const int qs = p.q_start[r], n = p.q_start[r + 1] - qs;
+  if (n <= 0) return;
+  const int start = p.ctx_len[r] - n;
+  const int bi = (n + per_block - 1) / per_block - 1 - rows_x;
+  if (bi < 0) return;
+  const int g = p.nh / p.nkv;
+  const int t0 = bi * per_block + wave * p.tpw;
+  const int ntok = max(0, min(p.tpw, n - t0));
+  const int tok = lr / g, hq = lr - tok * g;
+  if (tok >= ntok) return;
+  const int blk_lo = start + bi * per_block, blk_hi = start + min(n, (bi + 1) * per_block) - 1;
+  const int key_lo = p.window > 0 ? max(0, blk_lo - p.window + 1) : 0;
+  const int ranges = (blk_hi / 32 - key_lo / 32) / p.chunk + 1;
+  const size_t slot0 = ((((size_t)blockIdx.z * p.nkv + kvh) * row_blocks + rows_x) * p.nchunks) * 4 + wave;
+  float m = -INFINITY;
+  for (int c = 0; c < ranges; c++) m = fmaxf(m, p.part_ml[(slot0 + (size_t)c * 4) * 128 + lr]);
+  f32x4 acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float l = 0.f;
+  for (int c = 0; c < ranges; c++) {
+    const size_t slot = slot0 + (size_t)c * 4;
+    const float mc = p.part_ml[slot * 128 + lr];
+    const float w = mc == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mc - m);
+    l += w * p.part_ml[slot * 128 + 32 + lr];
+    const f32x4* po = (const f32x4*)p.part_o + slot * ((size_t)dts * 4 * 64) + (size_t)dt * 4 * 64 + lane;
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[j] += w * po[j * 64];
+  }
+  const float inv = 1.f / l;
+  __bf16* orow = p.out + ((size_t)(qs + t0 + tok) * p.nh + kvh * g + hq) * p.hd;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int d = dt * 32 + 8 * j + 4 * lk;
+    if (d < p.hd) {
+      bf16x4 w4;
+#pragma unroll
+      for (int i = 0; i < 4; i++) w4[i] = (__bf16)(acc[j][i] * inv);
+      *(bf16x4*)(orow + d) = w4;
+    }
+  }
 }
 
 // One wave per (request, KV head, chunk of 64 keys) for requests that bring one token.
@@ -896,44 +981,84 @@ static int launch_attn(const AttnParams& p, dim3 grid, hipStream_t s) {
   return zk_launch_status("zk_attention_bf16");
 }
 
-template <int HD16, int NW>
+template <int HD16, int NW, bool SPLIT>
 static int launch_shared_one(const AttnParams& p, dim3 grid, hipStream_t s) {
   constexpr int HD = HD16 * 16;
   constexpr size_t lds = ((size_t)2 * 32 * (HD + 8) + (size_t)2 * HD * (32 + 8)) * sizeof(__bf16);
   static bool prepared = false;
   if (!prepared) {
-    if (lds > 64 * 1024 && hipFuncSetAttribute((const void*)attn_shared_kernel<HD16, NW>,
+    if (lds > 64 * 1024 && hipFuncSetAttribute((const void*)attn_shared_kernel<HD16, NW, SPLIT>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return zk_fail("zk_attention_bf16: the shared-tile kernel's LDS buffers were refused");
     prepared = true;
   }
-  attn_shared_kernel<HD16, NW><<<grid, NW * 64, lds, s>>>(p);
+  attn_shared_kernel<HD16, NW, SPLIT><<<grid, NW * 64, lds, s>>>(p);
   return zk_launch_status("zk_attention_bf16 (shared tiles)");
 }
 
-template <int NW>
+template <int NW, bool SPLIT>
 static int launch_shared(const AttnParams& p, dim3 grid, hipStream_t s) {
   switch (p.hd / 16) {
-    case 1: return launch_shared_one<1, NW>(p, grid, s);
-    case 2: return launch_shared_one<2, NW>(p, grid, s);
-    case 4: return launch_shared_one<4, NW>(p, grid, s);
-    case 8: return launch_shared_one<8, NW>(p, grid, s);
+    case 1: return launch_shared_one<1, NW, SPLIT>(p, grid, s);
+    case 2: return launch_shared_one<2, NW, SPLIT>(p, grid, s);
+    case 4: return launch_shared_one<4, NW, SPLIT>(p, grid, s);
+    case 8: return launch_shared_one<8, NW, SPLIT>(p, grid, s);
     case 16:
-      if constexpr (NW <= 4) return launch_shared_one<16, NW>(p, grid, s);
+      if constexpr (NW <= 4) return launch_shared_one<16, NW, SPLIT>(p, grid, s);
       else return zk_fail("zk_attention_bf16: eight waves a block take head sizes up to 128");
     default: return zk_fail("zk_attention_bf16: head_dim must be 16, 32, 64, 128 or 256");
   }
 }
 
+// Bytes the portions' split variant needs behind the decoded tokens' part of the workspace.
+// Per (request, KV head, block of rows, range, wave): the wave's accumulators as they lie in
+// its registers (ceil(hd / 32) x 16 floats a lane) and 128 floats of maxima and sums.
+static size_t portion_split_bytes(long row_blocks, int nkv, int hd, int ranges) {
+  const size_t dt = (size_t)(hd + 31) / 32;
+  return (size_t)row_blocks * nkv * ranges * 4 * (dt * 16 * 64 + 128) * sizeof(float);
+}
+
+// The ranges of keys for a launch of few blocks of rows: tiles a range (0: do not split) and the
+// most ranges a block of rows can have.  Priced for one causal request of max_q_len rows ending
+// at max_ctx, window or not: blocks(ct) = sum over the blocks of rows of ceil(tiles / ct), and
+// the time goes with ceil(blocks / 256) * ct; of equal times the longer range (fewer partial
+// results).  No split unless it at least halves the longest block's tiles; at most
+// ATT_MOST_RANGES ranges for the longest block of rows the caller's limits allow (bound_tiles),
+// which bounds the workspace.
+static int portion_ranges(int max_q_len, int max_ctx, int window, int per_block, int nkv, int r_prefill,
+                          int bound_tiles) {
+  const int row_blocks = (max_q_len + per_block - 1) / per_block;
+  auto tiles_of = [&](int bi) {
+    const int lo = max_ctx - max_q_len + bi * per_block, hi = std::min(max_ctx, lo + per_block) - 1;
+    const int klo = window > 0 ? std::max(0, lo - window + 1) : 0;
+    return hi / 32 - klo / 32 + 1;
+  };
+  int longest = 0;
+  for (int bi = 0; bi < row_blocks; bi++) longest = std::max(longest, tiles_of(bi));
+  static const int cands[] = {32, 24, 16, 12, 10, 8, 6, 4};
+  int best = 0;
+  long best_cost = (long)((long)row_blocks * nkv * r_prefill + 255) / 256 * longest;
+  for (int ct : cands) {
+    if (2 * ct > longest || (bound_tiles + ct - 1) / ct > ATT_MOST_RANGES) continue;
+    long blocks = 0;
+    for (int bi = 0; bi < row_blocks; bi++) blocks += (tiles_of(bi) + ct - 1) / ct;
+    blocks *= (long)nkv * r_prefill;
+    const long cost = (blocks + 255) / 256 * ct + 4;          // + the joining launch, in tiles' worth
+    if (cost < best_cost) { best = ct; best_cost = cost; }
+  }
+  return best;
+}
+
 // 0: the portion kernel is chosen by the sizes; 1: a group of rows a block; 4, 8: shared
-// tiles with that many waves a block.  For tests and measurements (process-wide).
+// tiles with that many waves a block; 5: shared tiles, four waves, the keys in ranges (as far as
+// the workspace allows).  For tests and measurements (process-wide).
 static int portion_kernel_mode = 0;
 
 extern "C" {
 
 int zk_attention_bf16_portion_kernel(int mode) {
   const int before = portion_kernel_mode;
-  if (mode == 0 || mode == 1 || mode == 4 || mode == 8) portion_kernel_mode = mode;
+  if (mode == 0 || mode == 1 || mode == 4 || mode == 5 || mode == 8) portion_kernel_mode = mode;
   return before;
 }
 
@@ -949,6 +1074,15 @@ int zk_attention_bf16_supports(int nh, int nkv, int hd, int bs) {
 size_t zk_attention_bf16_workspace(int n_decode, int nh, int hd, int max_ctx) {
   const size_t nchunks = ((size_t)max_ctx + ATT_CHUNK - 1) / ATT_CHUNK;      // an upper bound for both variants
   return (size_t)n_decode * nh * nchunks * (hd + 2) * sizeof(float);
+}
+
+// Bytes of workspace that let portions of up to ``max_rows`` rows in all split their keys into
+// ranges (a launch of few blocks of rows with long contexts), on top of the decoded tokens'
+// part.  A caller that brings less gets the kernels that need none.
+size_t zk_attention_bf16_portion_workspace(int max_rows, int nh, int nkv, int hd) {
+  if (max_rows <= 0 || nkv <= 0 || nh % nkv || hd <= 0) return 0;
+  const int per_block = 4 * std::max(1, 32 / (nh / nkv));
+  return portion_split_bytes((max_rows + per_block - 1) / per_block, nkv, hd, ATT_MOST_RANGES) + 256;
 }
 
 // Whether decoded tokens of these sizes run on the 16-wide tiles (partial results joined four
@@ -1031,9 +1165,48 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
       else if (single >= 768) shared_waves = 4;
       if (shared_waves == 8 && hd > 128) shared_waves = 4;       // no room for two waves a SIMD
     }
-    if (shared_waves) {
+    // Few blocks of rows with many keys each (a portion of a few hundred rows behind thousands of
+    // tokens): four groups a block and the keys in ranges, where the workspace behind the decoded
+    // tokens' part holds the ranges' partial results.  512 rows behind 3,584 tokens, 8 heads of
+    // 256: 111 -> 52 us; behind 7,680: 209 -> 79 us; 16 heads of 256: 118 -> 76 us; 32 heads of
+    // 128: 100 -> 73 us.  A whole prompt from its first token (1,024 or 2,048 rows of 8 heads of
+    // 256) takes the same time either way: its blocks of rows are many and short already.
+    int range_tiles = 0, most_ranges = 0;
+    size_t split_at = 0;
+    if (bs >= 8 && (portion_kernel_mode == 5 || (portion_kernel_mode == 0 && !shared_waves))) {
+      const int per_block = 4 * p.tpw;
+      // no block of rows has more tiles than this, whatever its request's length
+      int bound = (max_ctx + 31) / 32;
+      if (window > 0) bound = std::min(bound, (window + per_block + 31) / 32 + 1);
+      range_tiles = portion_ranges(max_q_len, max_ctx, window, per_block, nkv, r_prefill, bound);
+      if (range_tiles) {
+        most_ranges = (bound + range_tiles - 1) / range_tiles;
+        if (R - r_prefill > 0) split_at = (zk_attention_bf16_workspace(R - r_prefill, nh, hd, max_ctx) + 255) / 256 * 256;
+        const size_t need = portion_split_bytes((long)r_prefill * ((max_q_len + per_block - 1) / per_block), nkv, hd,
+                                                most_ranges);
+        if (workspace == nullptr || (uintptr_t)workspace % 16 != 0 || split_at + need > workspace_bytes)
+          range_tiles = 0;
+      }
+    }
+    if (range_tiles) {
+      const int per_block = 4 * p.tpw;
+      AttnParams ps = p;
+      ps.chunk = range_tiles;
+      ps.nchunks = most_ranges;
+      const int row_blocks = (max_q_len + per_block - 1) / per_block;
+      const size_t slots = (size_t)r_prefill * nkv * row_blocks * most_ranges * 4;
+      const int dts = (hd + 31) / 32;
+      ps.part_o = (float*)((char*)workspace + split_at);
+      ps.part_ml = ps.part_o + slots * dts * 16 * 64;
+      dim3 grid(row_blocks * most_ranges, nkv, r_prefill);
+      rc = launch_shared<4, true>(ps, grid, s);
+      if (rc) return rc;
+      attn_portion_join_kernel<<<dim3(row_blocks * 4 * dts, nkv, r_prefill), 64, 0, s>>>(ps, per_block, row_blocks, dts);
+      rc = zk_launch_status("zk_attention_bf16 (join of the portions' ranges)");
+    } else if (shared_waves) {
+      if (shared_waves == 5) shared_waves = 4;
       dim3 grid((groups + shared_waves - 1) / shared_waves, nkv, r_prefill);
-      rc = shared_waves == 4 ? launch_shared<4>(p, grid, s) : launch_shared<8>(p, grid, s);
+      rc = shared_waves == 4 ? launch_shared<4, false>(p, grid, s) : launch_shared<8, false>(p, grid, s);
     } else if (single > 256 && paired <= 256) rc = launch_attn<false, true>(p, dim3((groups + 1) / 2, nkv, r_prefill), s);
     else rc = launch_attn<false, false>(p, dim3(groups, nkv, r_prefill), s);
     if (rc) return rc;

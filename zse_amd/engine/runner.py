@@ -16,6 +16,8 @@ HIP graph per batch size as there (model_runner.py:1806-1932).
 """
 from __future__ import annotations
 
+import inspect
+
 import weakref
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
@@ -198,8 +200,11 @@ class StepRunner:
         # what it needs at this runner's limits, and refuses limits it cannot serve, here
         need = 0
         for part in model.parts():
-            need = max(need, int(part.prepare(self.k, self.dtype, self.max_seqs, self.max_model_len,
-                                              self.page_size)))
+            limits = (self.k, self.dtype, self.max_seqs, self.max_model_len, self.page_size)
+            if "max_batch_tokens" in inspect.signature(part.prepare).parameters:
+                need = max(need, int(part.prepare(*limits, max_batch_tokens=self.max_batch_tokens)))
+            else:
+                need = max(need, int(part.prepare(*limits)))
         try:
             self.workspace = rt.zeros((max(need // 4 + 1, 64),), F32)
         except Exception as e:

@@ -59,13 +59,15 @@ class PagedAttention(Part):
         s = self.spec
         return PagedKV(s.num_kv_heads, s.head_dim, s.window)
 
+    PORTION_RANGES_BYTES = 192 << 20
+
     def wants_v_transposed(self, kernels, dtype: str, page_size: int) -> bool:
         """The matrix-core kernel reads V as [page][kv head][hd][bs]."""
         s = self.spec
         return bool(dtype == BF16 and kernels.has("zk_attention_bf16") and
                     kernels.zk_attention_bf16_supports(s.num_heads, s.num_kv_heads, s.head_dim, page_size))
 
-    def prepare(self, kernels, dtype, max_seqs, max_model_len, page_size) -> int:
+    def prepare(self, kernels, dtype, max_seqs, max_model_len, page_size, max_batch_tokens=0) -> int:
         """Workspace of the split attention of decoded tokens at the runner's limits, and the
         number of keys a wave of it takes.  That number fixes where the sums over keys are cut:
         it follows from the limits alone, never from a step's batch, so a request's result does
@@ -81,8 +83,15 @@ class PagedAttention(Part):
             raise ValueError(f"attention with {s.num_heads} heads, {s.num_kv_heads} KV heads of "
                              f"{s.head_dim}: the longest context its decode kernel takes is {longest} "
                              f"tokens, the runner asks for {max_model_len}")
-        return int(kernels.zk_attention_bf16_workspace(int(max_seqs), s.num_heads, s.head_dim,
-                                                       int(max_model_len)))
+        need = int(kernels.zk_attention_bf16_workspace(int(max_seqs), s.num_heads, s.head_dim, int(max_model_len)))
+        # room for a launch of few, long portions to cut its keys into ranges: as much as a step's
+        # tokens can ask for, but no more than PORTION_RANGES_BYTES (a launch that would need more
+        # has blocks enough without the ranges, or runs on the kernels that need no workspace)
+        if max_batch_tokens > 0 and kernels.has("zk_attention_bf16_portion_workspace"):
+            extra = int(kernels.zk_attention_bf16_portion_workspace(int(max_batch_tokens), s.num_heads, s.num_kv_heads,
+                                                                    s.head_dim))
+            need = (need + 255) // 256 * 256 + min(extra, self.PORTION_RANGES_BYTES)
+        return need
 
     def forward(self, ctx, x: Tensor, cache) -> Tensor:
         s, k = self.spec, ctx.k

@@ -68,11 +68,14 @@ class Part:
     def children(self) -> List["Part"]:
         return []
 
-    def prepare(self, kernels, dtype: str, max_seqs: int, max_model_len: int, page_size: int) -> int:
+    def prepare(self, kernels, dtype: str, max_seqs: int, max_model_len: int, page_size: int,
+                max_batch_tokens: int = 0) -> int:
         """Called once by the step runner, with its limits, before the first step.  A part
         fixes here whatever must not change from step to step, refuses limits its kernels
         cannot serve (with the numbers, at construction and not in the middle of a run) and
-        returns the bytes of the runner's shared workspace its kernels need for one launch."""
+        returns the bytes of the runner's shared workspace its kernels need for one launch.
+        ``max_batch_tokens``: the most tokens a step brings (0: not said); a part whose
+        ``prepare`` does not take it is called without."""
         return 0
 
 

@@ -205,6 +205,9 @@ class KernelLibrary:
             self._dll.zk_attention_bf16_max_context.restype = C.c_longlong
             self._dll.zk_attention_bf16_max_context.argtypes = [_I, _I, _I, _I]
             self.zk_attention_bf16_max_context = self._dll.zk_attention_bf16_max_context
+            self._dll.zk_attention_bf16_portion_workspace.restype = C.c_size_t
+            self._dll.zk_attention_bf16_portion_workspace.argtypes = [_I, _I, _I, _I]
+            self.zk_attention_bf16_portion_workspace = self._dll.zk_attention_bf16_portion_workspace
             self._dll.zk_attention_bf16_portion_kernel.restype = C.c_int
             self._dll.zk_attention_bf16_portion_kernel.argtypes = [_I]
             self.zk_attention_bf16_portion_kernel = self._dll.zk_attention_bf16_portion_kernel
