@@ -1037,13 +1037,13 @@ static int portion_ranges(int max_q_len, int max_ctx, int window, int per_block,
   for (int bi = 0; bi < row_blocks; bi++) longest = std::max(longest, tiles_of(bi));
   static const int cands[] = {32, 24, 16, 12, 10, 8, 6, 4};
   int best = 0;
-  long best_cost = (long)((long)row_blocks * nkv * r_prefill + 255) / 256 * longest;
+  long best_cost = (long)((long)row_blocks * nkv * r_prefill + 255) / 256 * (longest + 10);
   for (int ct : cands) {
     if (2 * ct > longest || (bound_tiles + ct - 1) / ct > ATT_MOST_RANGES) continue;
     long blocks = 0;
     for (int bi = 0; bi < row_blocks; bi++) blocks += (tiles_of(bi) + ct - 1) / ct;
     blocks *= (long)nkv * r_prefill;
-    const long cost = (blocks + 255) / 256 * ct + 4;          // + the joining launch, in tiles' worth
+    const long cost = (blocks + 255) / 256 * (ct + 10) + 6;   // a block's start and end, the joining launch: in tiles' worth
     if (cost < best_cost) { best = ct; best_cost = cost; }
   }
   return best;
