@@ -637,9 +637,8 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
   if (!SPLIT && !row_ok) return;
   if (SPLIT) {
     // A wave's results of its range, as they lie in its registers: 16 bytes a lane, a wave's 64
-    // lanes one contiguous KB per (dt, j), so every store is whole lines (stored row by row, a
-    // lane's pieces are 32 bytes here and 32 there: measured three times slower).  The joining
-    // kernel reads them back with the same lanes.  Every lane stores, rows or not.
+    // lanes one contiguous KB per (dt, j), so every store is whole lines.  The joining kernel
+    // reads them back with the same lanes.  Every lane stores, rows or not.
     const size_t slot = ((((size_t)blockIdx.z * p.nkv + kvh) * (gridDim.x / p.nchunks) + rows_x) * p.nchunks + range) * NW + wave;
     p.part_ml[slot * 128 + lane] = lk == 0 ? m_run : l_run;
     f32x4* po = (f32x4*)p.part_o + slot * (DT * 4 * 64) + lane;
