@@ -1168,8 +1168,8 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
     // tokens): four groups a block and the keys in ranges, where the workspace behind the decoded
     // tokens' part holds the ranges' partial results.  512 rows behind 3,584 tokens, 8 heads of
     // 256: 111 -> 52 us; behind 7,680: 209 -> 79 us; 16 heads of 256: 118 -> 76 us; 32 heads of
-    // 128: 100 -> 73 us.  A whole prompt from its first token (1,024 or 2,048 rows of 8 heads of
-    // 256) takes the same time either way: its blocks of rows are many and short already.
+    // 128: 100 -> 73 us.  A whole prompt from its first token, 8 heads of 256: 2,048 rows 74 -> 62
+    // us, 1,024 rows the same time either way (its blocks of rows are many and short already).
     int range_tiles = 0, most_ranges = 0;
     size_t split_at = 0;
     if (bs >= 8 && (portion_kernel_mode == 5 || (portion_kernel_mode == 0 && !shared_waves))) {
