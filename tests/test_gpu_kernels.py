@@ -454,6 +454,57 @@ def test_attention_over_pages(rt, kernel, case):
         assert np.array_equal(outs[0], outs[turns.index((64, 5))]) and not np.array_equal(outs[0], outs[turns.index((64, 4))])
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_portion_attention_kernels_agree_on_random_launches(rt, seed):
+    """Random launches (one to three portions of 2 to 700 rows behind 0 to 1,500 tokens, up to two
+    decoded tokens beside them, 1 to 16 heads a KV head, windows, caps, pages of 8 to 64 keys,
+    pages in random order): the kernels with shared tiles (four waves, eight, with the keys in
+    ranges, and the choice by size) against the kernel of one group a block, which the cases above
+    hold against NumPy."""
+    k = rt.kernels("bfloat16")
+    rng = np.random.default_rng(1000 + seed)
+    nkv, g = int(rng.choice([1, 2, 3, 4, 8])), int(rng.choice([1, 2, 3, 4, 5, 8, 16]))
+    nh, hd, bs = nkv * g, int(rng.choice([16, 32, 64, 128, 256])), int(rng.choice([8, 16, 32, 64]))
+    reqs = [(int(rng.integers(0, 1500)), int(rng.integers(2, 700))) for _ in range(int(rng.integers(1, 4)))]
+    n_multi = len(reqs)
+    reqs += [(int(rng.integers(1, 1200)), 1) for _ in range(int(rng.integers(0, 3)))]
+    window, cap = int(rng.choice([0, 0, 40, 300, 1000])), float(rng.choice([0.0, 30.0, 50.0]))
+    total = [a + b for a, b in reqs]
+    max_blocks = max(-(-t // bs) for t in total) + 1
+    pages = sum(-(-t // bs) for t in total) + 2
+    KC, VC = rt.empty((pages, nkv, bs, hd), "bfloat16"), rt.empty((pages, nkv, hd, bs), "bfloat16")
+    k.zk_fill_normal(KC.ptr, 1, KC.numel, 1, 3 * seed + 1, 0.0, 1.0, rt.stream)
+    k.zk_fill_normal(VC.ptr, 1, VC.numel, 1, 3 * seed + 2, 0.0, 1.0, rt.stream)
+    table, free = np.full((len(reqs), max_blocks), -1, np.int32), list(rng.permutation(pages))
+    for r, t in enumerate(total):
+        for j in range(-(-t // bs)):
+            table[r, j] = free.pop()
+    T = sum(n for _, n in reqs)
+    qs = np.concatenate([[0], np.cumsum([n for _, n in reqs])]).astype(np.int32)
+    TBL, QS, CL = rt.upload(table), rt.upload(qs), rt.upload(np.array(total, np.int32))
+    Q = rt.empty((T, nh * hd), "bfloat16")
+    k.zk_fill_normal(Q.ptr, 1, Q.numel, 1, 3 * seed + 3, 0.0, 1.0, rt.stream)
+    max_q, max_ctx = max(n for _, n in reqs), -(-max(total) // 256) * 256
+    ws_bytes = (k.zk_attention_bf16_workspace(len(reqs), nh, hd, max_ctx) + 255) // 256 * 256
+    ws_bytes += k.zk_attention_bf16_portion_workspace(n_multi * (max_q + 128), nh, nkv, hd)
+    ws = rt.zeros((ws_bytes // 4 + 16,), "float32")
+    outs = {}
+    for mode in (1, 4, 8, 5, 0):
+        OUT = rt.zeros((T, nh * hd), "bfloat16")
+        k.zk_attention_bf16_portion_kernel(mode)
+        try:
+            k.zk_attention_bf16(Q.ptr, nh * hd, KC.ptr, VC.ptr, TBL.ptr, max_blocks, QS.ptr, CL.ptr, OUT.ptr, len(reqs),
+                                n_multi, max_q, max_ctx, nh, nkv, hd, bs, hd ** -0.5, cap, window, 64, ws.ptr,
+                                ws.nbytes, rt.stream)
+        finally:
+            k.zk_attention_bf16_portion_kernel(0)
+        outs[mode] = rt.download_f32(OUT)
+    for mode in (4, 8, 5, 0):
+        assert np.isfinite(outs[mode]).all()
+        err = np.abs(outs[mode] - outs[1]).max()
+        assert err <= 0.02 * max(1.0, np.abs(outs[1]).max()), f"kernel {mode}: {err}; {nh} heads, {nkv} KV heads of {hd}, {reqs}"
+
+
 def run_attention(rt, kernel, q, kk, vv, past, nh, nkv, hd, bs, scale, cap, window, chunk=64, max_ctx=None):
     """One request holding ``past`` cached tokens brings the rest of ``kk``/``vv`` [ctx, nkv, hd]
     with queries ``q`` [n, nh, hd]; pages are laid out in order.  Returns [n, nh, hd]."""
