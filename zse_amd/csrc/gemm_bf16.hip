@@ -543,21 +543,50 @@ __global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_t
     for (int i = 0; i < BPT; i++) *(bf16x8*)(&tiles[buf * (BM + BN) + BM + brow[i]][bcol]) = rb[i];
   };
   auto multiply = [&](int buf) {
+    if constexpr (NWM * NWN > 8) {
+      // sixteen waves: 128 registers a wave, no room for a second set of operands
 #pragma unroll
-    for (int ks = 0; ks < GT_BK / 16; ks++) {
-      bf16x8 fa[WMT], fb[2];
+      for (int ks = 0; ks < GT_BK / 16; ks++) {
+        bf16x8 fa[WMT], fb[2];
 #pragma unroll
-      for (int i = 0; i < WMT; i++) fa[i] = *(const bf16x8*)(&tiles[buf * (BM + BN) + wm * (32 * WMT) + i * 32 + lr][ks * 16 + lk * 8]);
+        for (int i = 0; i < WMT; i++) fa[i] = *(const bf16x8*)(&tiles[buf * (BM + BN) + wm * (32 * WMT) + i * 32 + lr][ks * 16 + lk * 8]);
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          const int row = GATED ? j * (BN / 2) + wn * 32 : wn * 64 + j * 32;
+          fb[j] = *(const bf16x8*)(&tiles[buf * (BM + BN) + BM + row + lr][ks * 16 + lk * 8]);
+        }
+#pragma unroll
+        for (int i = 0; i < WMT; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+      }
+      return;
+    }
+    // the operands of k step ks + 1 are read from LDS while the products of step ks run: two
+    // sets of fragments, and a fence that keeps the reads before the products they follow in
+    // the source (the compiler would put every read right before its use and wait for it)
+    bf16x8 fa[2][WMT], fb[2][2];
+    auto read = [&](int ks, bf16x8 (&a)[WMT], bf16x8 (&b)[2]) {
+#pragma unroll
+      for (int i = 0; i < WMT; i++) a[i] = *(const bf16x8*)(&tiles[buf * (BM + BN) + wm * (32 * WMT) + i * 32 + lr][ks * 16 + lk * 8]);
 #pragma unroll
       for (int j = 0; j < 2; j++) {
         const int row = GATED ? j * (BN / 2) + wn * 32 : wn * 64 + j * 32;
-        fb[j] = *(const bf16x8*)(&tiles[buf * (BM + BN) + BM + row + lr][ks * 16 + lk * 8]);
+        b[j] = *(const bf16x8*)(&tiles[buf * (BM + BN) + BM + row + lr][ks * 16 + lk * 8]);
       }
+    };
+    read(0, fa[0], fb[0]);
+#pragma unroll
+    for (int ks = 0; ks < GT_BK / 16; ks++) {
+      if (ks + 1 < GT_BK / 16) read(ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0x616);
 #pragma unroll
       for (int i = 0; i < WMT; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks & 1][j], fa[ks & 1][i], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0x616);
     }
   };
   // The loop takes two tiles a turn.  An odd number of tiles: when EXACT the first tile is
