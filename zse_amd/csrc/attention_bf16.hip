@@ -481,36 +481,52 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
   // [8c, 8c + 8) of channel d in part q / (HD tk / 8), d = (q / (tk / 8)) % HD, c = q % (tk / 8).
   const int tk_shift = min(bsh, 5);                     // log2 of a page's keys in a tile
   const int cpp_shift = tk_shift - 3;                   // log2 of the pieces of a channel in a page's part
-  int k_key[PPT], k_col[PPT], v_d[PPT], v_key[PPT];
+  // What does not change from tile to tile is worked out here, per piece: its place in the page
+  // table relative to the tile's first entry, its offset inside a page's block of the cache (the
+  // KV head, the key's place in the page, the channels) and its place in LDS.  A tile then costs
+  // a piece one table entry and one multiply-add.  (Tiles start at multiples of 32 keys: with
+  // pages of up to 32 keys a key's place in its page does not depend on the tile, with larger
+  // pages the whole tile lies in one page and the tile's offset in it is the same for all.)
+  int k_idx[PPT], v_idx[PPT], k_lds[PPT], v_lds[PPT];
+  unsigned k_off[PPT], v_off[PPT];
 #pragma unroll
   for (int j = 0; j < PPT; j++) {
     const int q = min(tid + j * NT, PIECES - 1);
-    k_key[j] = q / CPK;
-    k_col[j] = (q % CPK) * 8;
+    const int kk = q / CPK, col = (q % CPK) * 8;
     const int part = q / (HD << cpp_shift), rem = q - part * (HD << cpp_shift);
-    v_d[j] = rem >> cpp_shift;
-    v_key[j] = (part << tk_shift) + ((rem & ((1 << cpp_shift) - 1)) << 3);
+    const int d = rem >> cpp_shift;
+    const int vk = (part << tk_shift) + ((rem & ((1 << cpp_shift) - 1)) << 3);
+    k_idx[j] = kk >> bsh;
+    k_off[j] = (unsigned)(((kvh << bsh) + (kk & bmask)) * HD + col);
+    k_lds[j] = kk * KLD + col;
+    v_idx[j] = vk >> bsh;
+    v_off[j] = (unsigned)(((kvh * HD + d) << bsh) + (vk & bmask));
+    // keys 8c + (0..3) go to piece 2h of the channel, keys 8c + 4 + (0..3) to piece 2h + 1,
+    // both at slot 4 (c % 2), with h = c / 2
+    const int c = vk >> 3;
+    v_lds[j] = d * VLD + (c >> 1) * 16 + (c & 1) * 4;
   }
+  const size_t page_elems = ((size_t)nkv * HD) << bsh;        // of a page of K, and of a page of V
+  const int last_entry = p.max_blocks - 1;
   struct Pages { int k[PPT], v[PPT]; };
   struct Stage { bf16x8 k[PPT], v[PPT]; };
-  // a key past the block's last reads that one again (it is masked), a piece of V past it the
-  // piece the last key lies in: every address stays inside the request's pages
+  // A key past the request's last (in its last tile, or in the tile fetched after the last) is
+  // read from wherever its table entry points, page 0 where there is none: it is masked, and
+  // the cache holds finite values everywhere.
   auto look_up = [&](int key0, Pages& pg) {
+    const int first = key0 >> bsh;
 #pragma unroll
     for (int j = 0; j < PPT; j++) {
-      pg.k[j] = table[min(key0 + k_key[j], key_hi) >> bsh];
-      pg.v[j] = table[min(key0 + v_key[j], key_hi & ~7) >> bsh];
+      pg.k[j] = table[min(first + k_idx[j], last_entry)];
+      pg.v[j] = table[min(first + v_idx[j], last_entry)];
     }
   };
   auto fetch = [&](int key0, const Pages& pg, Stage& st) {
+    const unsigned in_page = (unsigned)(key0 & bmask);
 #pragma unroll
     for (int j = 0; j < PPT; j++) {
-      const int kk = min(key0 + k_key[j], key_hi);
-      st.k[j] = *(const bf16x8*)(p.kcache + ((((size_t)max(pg.k[j], 0) * nkv + kvh) << bsh) + (kk & bmask)) * HD +
-                                 k_col[j]);
-      const int kv = min(key0 + v_key[j], key_hi & ~7);
-      st.v[j] = *(const bf16x8*)(p.vcache + ((((size_t)max(pg.v[j], 0) * nkv + kvh) * HD + v_d[j]) << bsh) +
-                                 (kv & bmask));
+      st.k[j] = *(const bf16x8*)(p.kcache + ((size_t)max(pg.k[j], 0) * page_elems + (k_off[j] + in_page * HD)));
+      st.v[j] = *(const bf16x8*)(p.vcache + ((size_t)max(pg.v[j], 0) * page_elems + (v_off[j] + in_page)));
     }
   };
   auto stash = [&](int buf, const Stage& st) {
@@ -519,11 +535,8 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
 #pragma unroll
     for (int j = 0; j < PPT; j++) {
       if (PIECES % NT == 0 || tid + j * NT < PIECES) {
-        *(bf16x8*)(kb + k_key[j] * KLD + k_col[j]) = st.k[j];
-        // keys 8c + (0..3) go to piece 2h of the channel, keys 8c + 4 + (0..3) to piece 2h + 1,
-        // both at slot 4 (c % 2), with h = c / 2
-        const int c = v_key[j] >> 3;
-        __bf16* vrow = vb + v_d[j] * VLD + (c >> 1) * 16 + (c & 1) * 4;
+        *(bf16x8*)(kb + k_lds[j]) = st.k[j];
+        __bf16* vrow = vb + v_lds[j];
         bf16x4 lo4, hi4;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
