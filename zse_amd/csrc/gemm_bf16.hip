@@ -654,6 +654,31 @@ __global__ __launch_bounds__(256) void gemm_tile_join_kernel(
   tile_of_block(tile + tile_base, tiles_m, tiles_n, tm, tn);
   // float4 index of (tile, range p, wave, pair member j, lane, b): an accumulator is 4 float4
   const size_t per_wave = (size_t)WMT * 2 * 64 * 4;
+  if constexpr (!GATED) {
+    // A whole tile into a 16-bit C with rows of whole 16-byte pieces: a thread takes the two
+    // halves (lanes lr and lr + 32) of eight neighbouring columns of a row, so its store is 16
+    // bytes and four threads fill a 64-byte line (the general way below stores two bytes at a
+    // time, half a line's bytes from one wave and the other half from another).  The block's
+    // 256 threads are (b, lr, j) here; the sums are the same, in the same order.
+    const int m0 = tm * BM + (wave / NWN) * (32 * WMT) + i * 32, n0 = tn * BN + (wave % NWN) * 64;
+    if (!c_is_f32 && epi == EPI_NONE && ldc % 8 == 0 && (uintptr_t)C % 16 == 0 && m0 + 32 <= M && n0 + 64 <= N) {
+      const int lr = lane & 31, j = lane >> 5;
+      const f32x4* at = partials + ((size_t)tile * ksplit * NW + wave) * per_wave + ((size_t)(i * 2 + j) * 64 + lr) * 4 + b;
+      f32x4 lo = at[0], hi = at[32 * 4];
+      for (int p = 1; p < ksplit; p++) {
+        lo += at[(size_t)p * NW * per_wave];
+        hi += at[(size_t)p * NW * per_wave + 32 * 4];
+      }
+      bf16x8 out;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        out[e] = (__bf16)lo[e];
+        out[4 + e] = (__bf16)hi[e];
+      }
+      *(bf16x8*)((__bf16*)C + (size_t)(m0 + lr) * ldc + n0 + j * 32 + 8 * b) = out;
+      return;
+    }
+  }
   const f32x4* src = partials + ((size_t)tile * ksplit * NW + wave) * per_wave + ((size_t)(i * 2) * 64 + lane) * 4 + b;
   f32x4 x0 = src[0], x1 = src[64 * 4];
   for (int p = 1; p < ksplit; p++) {
