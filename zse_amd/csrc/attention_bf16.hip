@@ -1,7 +1,6 @@
 // Paged attention on the matrix cores, bfloat16 in, float softmax.
 //
-// One kernel serves prompt portions and decoded tokens.  A wave owns up to 32
-// query rows: TPW consecutive tokens of one request times the g = nh / nkv
+// A wave owns up to 32 query rows: TPW consecutive tokens of one request times the g = nh / nkv
 // query heads that share a KV head, so every K and V tile it loads serves the
 // whole group (the reference's paged_attention_v2 stages a K/V tile once for
 // the heads of a group too, orchestrator/kernels.py:687-854, but is never
@@ -19,6 +18,13 @@
 // h are keys 4h + e, slots e >= 4 are keys 8 + 4h + e - 4), and V is read with
 // the same permutation.  V is therefore cached transposed, [page][kv head][hd][bs],
 // so that four consecutive keys of a channel are one 8-byte load.
+//
+// Portions have three kernels, chosen by the launch's sizes (zk_attention_bf16): a group of 32
+// rows a block, its four waves sharing out the keys (attn_mfma_kernel: few groups); four or
+// eight consecutive groups a block with every tile of keys and values fetched once into LDS for
+// all of them (attn_shared_kernel: many groups); and the latter with the keys of a block of rows
+// cut into ranges over several blocks, joined by attn_portion_join_kernel (few groups with long
+// contexts: a portion of a prompt behind thousands of tokens).
 //
 // Decoded tokens use a split variant: the keys are cut into chunks of 64 (or 32, as
 // the caller says) aligned to absolute positions, one wave per chunk writes (max, sum, O)
