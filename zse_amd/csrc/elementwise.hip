@@ -441,8 +441,8 @@ __global__ __launch_bounds__(256) void rope_cache_write_token_kernel(
     }
   }
   // v heads.  Transposed cache: eight tokens in a row of the step whose slots are eight in a
-  // row of one page (a prompt portion) go out together, 8 values of a channel per store,
-  // from the block of the first of them; other tokens are written value by value.
+  // row of one page (a prompt portion) go out together, 8 values of a channel per store, each
+  // of the eight blocks an eighth of the channels; other tokens are written value by value.
   if (v_transposed) {
     const int tl = t - t % 8;
     bool together = bs % 8 == 0 && tl + 7 < (int)gridDim.x && slot_map != nullptr;
@@ -453,12 +453,14 @@ __global__ __launch_bounds__(256) void rope_cache_write_token_kernel(
       for (int e = 1; together && e < 8; e++) together = slot_map[tl + e] == slot0 + e;
     }
     if (together) {
-      if (t != tl) return;
+      // the eight tokens' blocks share the (kv head, channel) pairs among them, an eighth each
       typedef act_t av8 __attribute__((ext_vector_type(8)));
       const size_t page0 = slot0 / bs, off0 = slot0 % bs;
-      for (int it = tid; it < nkv * hd; it += 256) {
+      const act_t* row0 = qkv + (size_t)tl * (nh + 2 * nkv) * hd;
+      const int items = nkv * hd, mine = (items + 7) / 8, first = (t - tl) * mine;
+      for (int it = first + tid; it < min(first + mine, items); it += 256) {
         const int kvh = it / hd, d = it % hd;
-        const act_t* src = row + (size_t)(nh + nkv + kvh) * hd + d;
+        const act_t* src = row0 + (size_t)(nh + nkv + kvh) * hd + d;
         av8 v;
 #pragma unroll
         for (int e = 0; e < 8; e++) v[e] = src[(size_t)e * (nh + 2 * nkv) * hd];
