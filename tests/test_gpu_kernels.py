@@ -192,6 +192,39 @@ def test_gemm_bf16_layer_shapes_at_medium_rows(rt, N, K, gated):
         assert err < tol, f"M={M}: {err} against {tol}"
 
 
+@pytest.mark.parametrize("M,N,K,gated,cap", [(2048, 2304, 2048, False, 0.0), (1500, 8208, 2304, False, 0.0),
+                                              (4000, 9216, 2304, True, 0.0), (700, 14336, 3584, True, 0.0),
+                                              (2048, 4096, 2304, False, 30.0), (1027, 2320, 9216, False, 0.0),
+                                              (3000, 1168, 2304, True, 0.0)])
+def test_gemm_bf16_wide_blocks_with_strip_weights(rt, M, N, K, gated, cap):
+    """Thousands of rows against strip-layout weights with K a whole number of 64: the 128 x 256
+    and 256 x 256 blocks that copy their operands straight into LDS.  Row counts that end inside
+    a block, widths that end inside a block's columns (2320, 8208, gated 1168), a soft cap, K in
+    ranges with a join (1027 x 2320 x 9216), into a 16-bit C (whole blocks leave through LDS)
+    and into a 32-bit one, against the plain product of the same 16-bit inputs."""
+    k = rt.kernels("bfloat16")
+    rng = np.random.default_rng(M + N + K)
+    rows = 2 * N if gated else N
+    a, w = bf16(rng.normal(size=(M, K))), bf16(rng.normal(size=(rows, K)) * (0.02 if gated else 0.05))
+    A, W = up(rt, a, "bfloat16"), up(rt, w, "bfloat16")
+    WS = rt.empty(((rows + 15) // 16 * 16, K), "bfloat16")
+    k.zk_strip_layout(W.ptr, WS.ptr, rows, K, rt.stream)
+    ws = gemm_workspace(rt)
+    R = rt.empty((M, rows), "float32")
+    k.zk_gemm_plain(A.ptr, K, W.ptr, R.ptr, rows, 1, M, rows, K, rt.stream)
+    ref = rt.download(R).astype(np.float64)
+    want = gelu(ref[:, :N]) * ref[:, N:] if gated else (cap * np.tanh(ref / cap) if cap else ref)
+    epi = 2 if gated else (1 if cap else 0)
+    C32, C16 = rt.empty((M, N), "float32"), rt.empty((M, N), "bfloat16")
+    k.zk_gemm_bf16(A.ptr, K, WS.ptr, C32.ptr, N, 1, M, N, K, epi, cap, 1, ws.ptr, ws.nbytes, None, rt.stream)
+    k.zk_gemm_bf16(A.ptr, K, WS.ptr, C16.ptr, N, 0, M, N, K, epi, cap, 1, ws.ptr, ws.nbytes, None, rt.stream)
+    got32, got16 = rt.download(C32), rt.download_f32(C16)
+    tol = 2e-5 * math.sqrt(K) * max(1.0, np.abs(want).max())
+    assert np.abs(got32 - want).max() < tol
+    # the 16-bit C holds the 32-bit one's values, rounded once
+    assert np.array_equal(got16, bf16(got32))
+
+
 def test_gemm_bf16_random_shapes(rt):
     """Forty shapes drawn at random over the three kernels' ranges, both weight layouts, with
     and without the gated epilogue and the workspace: whatever the dispatch picks must agree

@@ -637,6 +637,156 @@ __global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_t
   tile_store<WMT, NWN, GATED>(acc, C, ldc, c_is_f32, M, N, m0, n0, wm, wn, lane, epi, cap);
 }
 
+// A tile product whose operands are copied from memory straight into LDS (global_load_lds, 16
+// bytes a lane): no registers hold a tile on its way and no LDS writes are issued, so a wave
+// has room for a second set of operand fragments, and LDS has room for GD_NS stages of 32 k
+// values each.  The block meets at a barrier once per stage, and the reads of a wave's operands
+// run one k step of 16 ahead of its products across that barrier: when the barrier of stage s
+// has shown that stage s + 1 is there, its first operands are read while the second half of
+// stage s is multiplied, so the matrix unit does not drain at a stage's end.  For weights in the
+// strip layout and K a whole number of 64; the sums and their order are those of
+// gemm_tile_kernel, and so are the partial sums of a split K and the results' way out.
+// Measured on 2B and 9B layer shapes of 2,048 and 4,096 rows against the 256 x 256 block of
+// sixteen waves that stages its tiles through registers: two stages of 64 k with one barrier
+// each and 16-byte pieces of sixteen different rows a quarter wave 1.05 of its time; the same
+// with 128-byte runs of a row 0.98; four stages of 32 k with the reads running ahead 0.96 (five
+// stages 0.97); eight waves of 128 x 64 each instead of sixteen of 64 x 64 0.94.
+//
+// Such a load puts lane l's 16 bytes at (destination + 16 l).  W: a strip's 1 KB for one k
+// step lies in LDS as it lies in memory, [k piece of 8][row 16][8 values]; an operand read
+// (row lane % 32, k piece lane / 32) takes whole 256-byte runs.  A: an instruction takes 16
+// rows x 32 k, four lanes a row (a 64-byte run of the row); lane c of a row fetches k piece
+// c ^ ((row / 4) % 4), so piece q of row R lies at place q ^ ((R / 4) % 4) of the row's 64
+// bytes and the sixteen rows a read takes at once lie in different banks.
+#define ZK_GLOBAL_AS __attribute__((address_space(1)))
+#define ZK_LDS_AS __attribute__((address_space(3)))
+#define GD_NS 4
+#define GD_BK 32
+template <int WMT, int NWM, int NWN, bool GATED>
+__global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_tile_direct_kernel(
+    const __bf16* __restrict__ A, int lda, const __bf16* __restrict__ W, void* __restrict__ C, int ldc,
+    int c_is_f32, int M, int N, int K_all, int epi, float cap, int tiles_m, int tiles_n, int w_strip,
+    f32x16* __restrict__ partials, int ksplit, int tile_base) {
+  constexpr int BM = 32 * WMT * NWM, BN = 64 * NWN, NW = NWM * NWN;
+  constexpr int LPA = BM / 16 / NW, LPB = BN / 16 / NW;     // row blocks of A, strips of W, a wave copies
+  static_assert(LPA * NW * 16 == BM && LPB * NW * 16 == BN, "the waves do not share the copies evenly");
+  constexpr int HALF = BM * GD_BK * 2, STAGE = (BM + BN) * GD_BK * 2;      // bytes of a stage's A part, of a stage
+  extern __shared__ __align__(16) unsigned char gt_lds[];
+  int tm, tn;
+  tile_of_block(blockIdx.x + tile_base, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM;
+  constexpr int NCOLS = GATED ? BN / 2 : BN;
+  const int n0 = tn * NCOLS;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / NWN, wn = wave % NWN;
+  const int lr = lane & 31, lk = lane >> 5;
+  const int ktiles = K_all / GT_BK;
+  const int kt0 = (int)((long)blockIdx.y * ktiles / ksplit), kt1 = (int)((long)(blockIdx.y + 1) * ktiles / ksplit);
+  const int ns = 2 * (kt1 - kt0);                       // stages: an even number
+  // a wave copies the 16-row blocks wave, wave + NW, .. of A and the same strips of W
+  const __bf16* ga[LPA];
+  const __bf16* gw[LPB];
+  const int ksteps = K_all / 32;
+  const int strips = GATED ? 2 * N / 16 : N / 16;
+#pragma unroll
+  for (int c = 0; c < LPA; c++) {
+    const int a_row = (wave + c * NW) * 16 + (lane >> 2);
+    ga[c] = A + (size_t)min(m0 + a_row, M - 1) * lda + (size_t)kt0 * GT_BK + (((lane & 3) ^ ((a_row >> 2) & 3)) * 8);
+  }
+#pragma unroll
+  for (int c = 0; c < LPB; c++) {
+    const int blk = wave + c * NW;
+    int gs;
+    if (GATED) gs = blk < BN / 32 ? n0 / 16 + blk : N / 16 + n0 / 16 + (blk - BN / 32);
+    else gs = n0 / 16 + blk;
+    gs = min(gs, strips - 1);
+    gw[c] = W + ((size_t)gs * ksteps + 2 * kt0) * 512 + lane * 8;
+  }
+  auto issue = [&](int buf, int stage) {
+    stage = min(stage, ns - 1);      // past the end: the last stage again, into a buffer nobody reads
+    unsigned char* dst = gt_lds + buf * STAGE + wave * 1024;
+#pragma unroll
+    for (int c = 0; c < LPA; c++)
+      __builtin_amdgcn_global_load_lds((const ZK_GLOBAL_AS void*)(ga[c] + (size_t)stage * GD_BK), (ZK_LDS_AS void*)(dst + c * NW * 1024), 16, 0, 0);
+#pragma unroll
+    for (int c = 0; c < LPB; c++)
+      __builtin_amdgcn_global_load_lds((const ZK_GLOBAL_AS void*)(gw[c] + (size_t)stage * 512), (ZK_LDS_AS void*)(dst + HALF + c * NW * 1024), 16, 0, 0);
+  };
+  // where a lane reads its operand pieces of k step ks (0 or 1) of a stage
+  int a_at[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ks++) a_at[ks] = (wm * (32 * WMT) + lr) * 64 + (((ks * 2 + lk) ^ ((lr >> 2) & 3)) * 16);   // + i * 2048
+  const int w_row = GATED ? wn * 32 : wn * 64;                                    // + j * (GATED ? 128 : 32)
+  const int w_at = HALF + (w_row / 16 + (lr >> 4)) * 1024 + lk * 256 + (lr & 15) * 16;   // + ks * 512 + j * W_J
+  constexpr int W_J = GATED ? (BN / 32) * 1024 : 2048;
+  f32x16 acc[WMT][2];
+#pragma unroll
+  for (int i = 0; i < WMT; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+  bf16x8 fa[2][WMT], fb[2][2];
+  auto read = [&](int buf, int ks) {
+    const unsigned char* base = gt_lds + buf * STAGE;
+#pragma unroll
+    for (int i = 0; i < WMT; i++) fa[ks][i] = *(const bf16x8*)(base + a_at[ks] + i * 2048);
+#pragma unroll
+    for (int j = 0; j < 2; j++) fb[ks][j] = *(const bf16x8*)(base + w_at + ks * 512 + j * W_J);
+  };
+  auto products = [&](int ks) {
+    __builtin_amdgcn_sched_barrier(0x616);
+#pragma unroll
+    for (int i = 0; i < WMT; i++)
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0x616);
+  };
+  // Stage s lives in buffer s % GD_NS.  In flight when a step begins: stages s + 1 .. s + GD_NS - 2
+  // (two loads a wave each); the wait is for the wave's own loads of stage s + 1, the barrier
+  // then says that every wave's are there and that every wave has read stage s - 1, whose buffer
+  // the next loads go to.
+  auto step = [&](int b, int s) {
+    read(b, 1);
+    products(0);
+    // (the barrier as text: before one it knows, the compiler waits for every load in flight)
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((LPA + LPB) * (GD_NS - 3)) : "memory");
+    issue((b + GD_NS - 1) % GD_NS, s + GD_NS - 1);
+    read((b + 1) % GD_NS, 0);
+    products(1);
+  };
+#pragma unroll
+  for (int b = 0; b < GD_NS - 1; b++) issue(b, b);
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((LPA + LPB) * (GD_NS - 2)) : "memory");
+  read(0, 0);
+  for (int s = 0; s < ns; s += GD_NS) {
+#pragma unroll
+    for (int b = 0; b < GD_NS; b += 2) {
+      if (b > 0 && s + b >= ns) break;
+      step(b, s + b);
+      step(b + 1, s + b + 1);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();                              // the buffers are free for the results' way out
+  if (ksplit > 1) {
+    f32x16* mine = partials + (((size_t)blockIdx.x * ksplit + blockIdx.y) * NW + wave) * (WMT * 2 * 64) + lane;
+#pragma unroll
+    for (int i = 0; i < WMT; i++)
+#pragma unroll
+      for (int j = 0; j < 2; j++) mine[(i * 2 + j) * 64] = acc[i][j];
+    return;
+  }
+  if (!c_is_f32 && m0 + BM <= M && n0 + NCOLS <= N && ldc % 8 == 0 && (uintptr_t)C % 16 == 0) {
+    constexpr int WCOLS = GATED ? 32 : 64;
+    tile_store_staged<WMT, GATED>(acc, (__bf16*)C, ldc, m0 + wm * (32 * WMT), n0 + wn * WCOLS, lane, epi, cap,
+                                  (__bf16*)gt_lds + (size_t)wave * (32 * WMT) * (WCOLS + 8));
+    return;
+  }
+  tile_store<WMT, NWN, GATED>(acc, C, ldc, c_is_f32, M, N, m0, n0, wm, wn, lane, epi, cap);
+}
+
 // Second half of a tile product whose K was split over blocks: the ranges are added in order.
 // A thread takes four consecutive floats of a lane's accumulator pair (i, 0), (i, 1), so the
 // partial sums are read in 16-byte pieces, neighbours by neighbouring threads.
@@ -689,17 +839,20 @@ __global__ __launch_bounds__(256) void gemm_tile_join_kernel(
                                    wave / NWN, wave % NWN, lane, epi, cap);
 }
 
-template <int WMT, int NWM, int NWN, bool GATED, bool EXACT>
+template <int WMT, int NWM, int NWN, bool GATED, bool EXACT, bool DIRECT = false>
 static int launch_tile(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M, int N,
                        int K, int epi, float cap, int w_strip, const GemmWorkspace& wsp, int ksplit,
                        int tail_split, hipStream_t s) {
   constexpr int BM = 32 * WMT * NWM, BN = 64 * NWN;
   constexpr int ncols = GATED ? BN / 2 : BN;
-  constexpr size_t lds = (size_t)2 * (BM + BN) * GT_LD * sizeof(__bf16);
+  constexpr size_t lds_staged = (size_t)2 * (BM + BN) * GT_LD * sizeof(__bf16);
+  constexpr size_t lds = DIRECT && (size_t)GD_NS * (BM + BN) * GD_BK * 2 > lds_staged ? (size_t)GD_NS * (BM + BN) * GD_BK * 2 : lds_staged;
+  auto kernel = gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT>;
+  if constexpr (DIRECT) kernel = gemm_tile_direct_kernel<WMT, NWM, NWN, GATED>;
   static bool prepared = false;
   if (!prepared) {
     if (lds > 64 * 1024 &&
-        hipFuncSetAttribute((const void*)gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT>,
+        hipFuncSetAttribute((const void*)kernel,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return zk_fail("zk_gemm_bf16: the tile kernel's LDS buffers were refused");
     prepared = true;
@@ -726,14 +879,14 @@ static int launch_tile(const void* A, int lda, const void* W, void* C, int ldc, 
   if (tail_split > 1 && (size_t)tail * tail_split * BM * BN * sizeof(float) > wsp.bytes)
     return wsp.too_small((size_t)tail * tail_split * BM * BN * sizeof(float));
   const int whole = tail_split > 1 ? tiles - tail : tiles;
-  gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT><<<dim3(whole, ksplit), 64 * NWM * NWN, lds, s>>>(
+  kernel<<<dim3(whole, ksplit), 64 * NWM * NWN, lds, s>>>(
       (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, tiles_m, tiles_n, w_strip,
       (f32x16*)ws, ksplit, 0);
   if (ksplit > 1)
     gemm_tile_join_kernel<WMT, NWM, NWN, GATED><<<dim3(tiles * WMT * NWM * NWN), 256, 0, s>>>(
         (const f32x4*)ws, ksplit, C, ldc, c_is_f32, M, N, epi, cap, tiles_m, tiles_n, 0, tiles);
   if (tail_split > 1) {
-    gemm_tile_kernel<WMT, NWM, NWN, GATED, EXACT><<<dim3(tail, tail_split), 64 * NWM * NWN, lds, s>>>(
+    kernel<<<dim3(tail, tail_split), 64 * NWM * NWN, lds, s>>>(
         (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, tiles_m, tiles_n, w_strip,
         (f32x16*)ws, tail_split, whole);
     gemm_tile_join_kernel<WMT, NWM, NWN, GATED><<<dim3(tail * WMT * NWM * NWN), 256, 0, s>>>(
@@ -1302,6 +1455,18 @@ static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc
     const size_t room = (wsp.ptr != nullptr && (uintptr_t)wsp.ptr % 64 == 0) ? wsp.split_bytes() : 0;
     tile_cost(TileChoice{variant, ksplit}, M, N, K, gated, room, &tail_split);
   }
+  // The two wide blocks have a form that copies its operands straight into LDS (weights in the
+  // strip layout, K a whole number of tiles): 3 to 6 % less time from about 200 rows on, the
+  // same sums in the same order.  (The 128 x 128 and 64 x 128 blocks gained nothing from it
+  // where K is split and lost where it is short.)
+#define ZK_DIRECT(W_, M_, N_)                                                                                              \
+  (gated ? launch_tile<W_, M_, N_, true, true, true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, wsp, ksplit, tail_split, s) \
+         : launch_tile<W_, M_, N_, false, true, true>(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, wsp, ksplit, tail_split, s))
+  if (w_strip && K % GT_BK == 0 && N % 16 == 0) {
+    if (variant == 3) return ZK_DIRECT(4, 2, 4);
+    if (variant == 2) return ZK_DIRECT(2, 2, 4);
+  }
+#undef ZK_DIRECT
   if (variant == 3) return gated ? ZK_TILE_(2, 4, 4, true, true) : ZK_TILE_(2, 4, 4, false, true);
   if (variant == 2) return ZK_TILE(2, 2, 4);
   if (variant == 1) return ZK_TILE(1, 2, 2);
