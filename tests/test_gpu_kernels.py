@@ -195,7 +195,9 @@ def test_gemm_bf16_layer_shapes_at_medium_rows(rt, N, K, gated):
 @pytest.mark.parametrize("M,N,K,gated,cap", [(2048, 2304, 2048, False, 0.0), (1500, 8208, 2304, False, 0.0),
                                               (4000, 9216, 2304, True, 0.0), (700, 14336, 3584, True, 0.0),
                                               (2048, 4096, 2304, False, 30.0), (1027, 2320, 9216, False, 0.0),
-                                              (3000, 1168, 2304, True, 0.0)])
+                                              (3000, 1168, 2304, True, 0.0),
+                                              # K of one and of two k tiles: fewer stages than LDS holds
+                                              (2500, 2304, 64, False, 0.0), (2100, 1024, 128, True, 0.0)])
 def test_gemm_bf16_wide_blocks_with_strip_weights(rt, M, N, K, gated, cap):
     """Thousands of rows against strip-layout weights with K a whole number of 64: the 128 x 256
     and 256 x 256 blocks that copy their operands straight into LDS.  Row counts that end inside
