@@ -745,9 +745,9 @@ __global__ __launch_bounds__(64 * NWM * NWN, NWM * NWN <= 4 ? 2 : 1) void gemm_t
   };
   // Stage s lives in buffer s % GD_NS.  In flight when a step begins: stages s + 1 .. s + GD_NS - 2
   // (LPA + LPB loads a wave each); the wait is for the wave's own loads of stage s + 1, the barrier
-  // then says that every wave's are there and that every wave has read stage s - 1 (its products
-  // of stage s, issued before the barrier, waited for every read before them), whose buffer the
-  // next loads go to.
+  // then says that every wave's are there and that every wave has read stage s - 1 (the products
+  // that use its operands were issued before the barrier, so the operands had arrived), whose
+  // buffer the next loads go to.
   auto step = [&](int b, int s) {
     read(b, 1);
     products(0);
