@@ -77,6 +77,9 @@ def test_window_release_rule():
         m.slot_mapping("r", 0, 12, 4)                     # a released page cannot be written
     sm = m.slot_mapping("r", 0, 21, 2)
     assert list(sm) == [t[5] * 4 + 1, t[5] * 4 + 2]
+    assert m.slot_of("r", 0, 22) == sm[1] and m.slot_of("r", 1, 3) == m.table("r", 1)[0] * 4 + 3
+    with pytest.raises(RuntimeError):
+        m.slot_of("r", 0, 15)                             # one position on a released page
     m.check()
 
 

@@ -259,3 +259,11 @@ def test_a_small_windowed_pool_is_what_runs_out():
         m.check()
     assert seen and not s.has_work() and all(len(r.output_tokens) == 12 for r in rs)
     assert all(p.free_pages == p.num_pages for p in m.pools)
+
+
+def test_tokens_at_is_a_slice_of_all_tokens():
+    r = Request("t", [1, 2, 3, 4], SamplingParams(max_tokens=8))
+    r.output_tokens = [10, 11, 12]
+    for start in range(7):
+        for count in range(0, 8 - start):
+            assert r.tokens_at(start, count) == r.all_tokens[start:start + count]

@@ -115,12 +115,15 @@ class CacheManager:
                              f"{self.max_model_len}")
         r = self._reqs[req]
         want = -(-upto // self.page_size)
-        need = [max(0, want - len(r.tables[g])) for g in range(len(self.groups))]
+        tables = r.tables
+        if all(len(t) >= want for t in tables):      # the usual case: the last page has room
+            return True
+        need = [max(0, want - len(t)) for t in tables]
         if any(need[g] > self.pools[g].free_pages for g in range(len(self.groups))):
             return False
         for g, n in enumerate(need):
             for _ in range(n):
-                r.tables[g].append(self.pools[g].alloc(req))
+                tables[g].append(self.pools[g].alloc(req))
         return True
 
     def commit(self, req, computed: int) -> List[List[int]]:
@@ -164,6 +167,13 @@ class CacheManager:
         t = self._reqs[req].tables[group]
         row[:len(t)] = t
         row[len(t):] = -1
+
+    def slot_of(self, req, group: int, pos: int) -> int:
+        """page * page_size + offset for one position (a decoded token's: no arrays)."""
+        page = self._reqs[req].tables[group][pos // self.page_size]
+        if page < 0:
+            raise RuntimeError(f"request {req!r}: a position to be written lies on a released page")
+        return page * self.page_size + pos % self.page_size
 
     def slot_mapping(self, req, group: int, start: int, n: int) -> np.ndarray:
         """page * page_size + offset for positions start .. start+n-1."""

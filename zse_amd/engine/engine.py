@@ -150,7 +150,7 @@ class Engine:
         if run >= 2:
             return self._decode_run(plan, run)
         entries = [StepEntry(s.request.request_id,
-                             s.request.all_tokens[s.start:s.start + s.count],
+                             s.request.tokens_at(s.start, s.count),
                              [s.count - 1] if s.sample else []) for s in plan.items]
         logits = self.runner.step(entries, download=False)
         rows = []
@@ -200,7 +200,7 @@ class Engine:
         pending, done, tokens_from = [], [], None
         for i in range(length):
             known = tokens_from is None
-            entries = [StepEntry(r.request_id, [r.all_tokens[s.start] if known else 0], [0])
+            entries = [StepEntry(r.request_id, [r.tokens_at(s.start, 1)[0] if known else 0], [0])
                        for r, s in zip(reqs, plan.items)]
             logits = runner.step(entries, download=False, tokens_from=tokens_from)
             ids = sampler.sample_deferred(logits, i)

@@ -31,7 +31,7 @@ class FinishReason(enum.Enum):
     ERROR = "error"       # the request cannot be served (it does not fit the cache alone)
 
 
-@dataclass
+@dataclass(eq=False)      # a request is itself: lists of requests are searched by identity, not by comparing every field
 class Request:
     request_id: object
     prompt_tokens: List[int]
@@ -52,6 +52,15 @@ class Request:
     @property
     def all_tokens(self) -> List[int]:
         return self.prompt_tokens + self.output_tokens
+
+    def tokens_at(self, start: int, count: int) -> List[int]:
+        """``all_tokens[start:start + count]`` without putting the two lists together."""
+        np_ = len(self.prompt_tokens)
+        if start + count <= np_:
+            return self.prompt_tokens[start:start + count]
+        if start >= np_:
+            return self.output_tokens[start - np_:start - np_ + count]
+        return self.prompt_tokens[start:] + self.output_tokens[:start + count - np_]
 
     @property
     def num_tokens(self) -> int:

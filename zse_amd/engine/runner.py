@@ -301,14 +301,22 @@ class StepRunner:
             e = entries[i]
             n = len(e.tokens)
             start = m.computed(e.req)
-            tokens[t:t + n] = np.asarray(e.tokens, dtype=np.int32)
-            positions[t:t + n] = np.arange(start, start + n, dtype=np.int32)
-            req_of_token[t:t + n] = r
+            if n == 1:          # a decoded token: numbers, no arrays
+                tokens[t] = e.tokens[0]
+                positions[t] = start
+                req_of_token[t] = r
+                for g in range(G):
+                    slot_maps[g][t] = m.slot_of(e.req, g, start)
+            else:
+                tokens[t:t + n] = np.asarray(e.tokens, dtype=np.int32)
+                positions[t:t + n] = np.arange(start, start + n, dtype=np.int32)
+                req_of_token[t:t + n] = r
+                for g in range(G):
+                    slot_maps[g][t:t + n] = m.slot_mapping(e.req, g, start, n)
             q_start[r] = t
             ctx_len[r] = start + n
             slot_of_req[r] = m.slot(e.req)
             for g in range(G):
-                slot_maps[g][t:t + n] = m.slot_mapping(e.req, g, start, n)
                 m.fill_table_row(e.req, g, tables[g][r])
             first_token[i] = t
             host_entries.append((e.req, m.slot(e.req), start, n))
