@@ -130,7 +130,8 @@ class StepRunner:
     def __init__(self, model: Model, rt: Runtime, dtype: str, page_size: int = 16,
                  num_pages: Optional[int] = None, cache_tokens: Optional[int] = None,
                  max_seqs: int = 64, max_batch_tokens: int = 4096, max_model_len: Optional[int] = None,
-                 tuned: Optional[bool] = None, use_graphs: bool = True, use_steplists: bool = True):
+                 tuned: Optional[bool] = None, use_graphs: bool = True, use_steplists: bool = True,
+                 graph_max_batch: int = 16):
         self.model, self.rt = model, rt
         self.dtype = canonical_dtype(dtype)
         if model.loaded_dtype != self.dtype:
@@ -141,6 +142,13 @@ class StepRunner:
             raise ValueError(f"the model was loaded with tuned={model_tuned}; the runner cannot run it with tuned={tuned}")
         self.tuned = model_tuned
         self.use_graphs = bool(use_graphs) and self.tuned
+        # Decode steps of more requests than this are launched from their launch lists instead:
+        # a graph is captured for a padded batch and the longest context it covers, and with
+        # many requests of uneven lengths its attention grids are mostly blocks that end at
+        # once, while a step of that size runs long enough to hide the launches of the next
+        # (192 requests, 64 live, 2B shapes: 51.1 -> 54.1 k tokens a second without graphs;
+        # steps of 1 to 16 requests of equal length take the same time either way).
+        self.graph_max_batch = int(graph_max_batch)
         self.page_size = int(page_size)
         self.max_seqs = int(max_seqs)
         self.max_batch_tokens = int(max_batch_tokens)
@@ -369,6 +377,8 @@ class StepRunner:
         (0: run eagerly).  Every entry brings one token and wants its logits."""
         if not self.use_graphs or not self.graph_safe:
             return 0
+        if len(entries) > self.graph_max_batch:
+            return 0
         if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
             return 0
         b = 1
@@ -484,10 +494,10 @@ class StepRunner:
             if e.req in seen:
                 raise ValueError(f"request {e.req!r} appears twice in one step")
             seen.add(e.req)
-            for tok in e.tokens:
-                if not (0 <= int(tok) < self.vocab):
-                    raise ValueError(f"request {e.req!r}: token id {tok} is outside the vocabulary "
-                                     f"of {self.vocab}")
+            lo, hi = min(e.tokens), max(e.tokens)
+            if not (0 <= int(lo) and int(hi) < self.vocab):
+                raise ValueError(f"request {e.req!r}: token id {lo if int(lo) < 0 else hi} is outside the "
+                                 f"vocabulary of {self.vocab}")
         T = sum(len(e.tokens) for e in entries)
         R = len(entries)
         if T > self.max_batch_tokens or R > self.max_seqs:
