@@ -665,7 +665,11 @@ def test_embed(rt, dtype, T, H, V):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("T,H,eps,uo", [(4, 96, 1e-5, 1), (3, 2304, 1e-6, 1), (2, 70, 1e-6, 0), (2, 9000, 1e-6, 1),
-                                        (3, 3584, 1e-6, 1), (2, 4608, 1e-6, 1), (2, 7000, 1e-6, 0)])
+                                        (3, 3584, 1e-6, 1), (2, 4608, 1e-6, 1), (2, 7000, 1e-6, 0),
+                                        # rows of 2,048 to 8,192 values in bfloat16: up to 64 of them
+                                        # take the kernel of 1,024 threads a row, more the one of 256
+                                        (8, 4096, 1e-6, 1), (64, 4608, 1e-6, 1), (65, 4608, 1e-6, 1), (5, 8192, 1e-5, 0),
+                                        (7, 2048, 1e-6, 1), (3, 2044, 1e-6, 1)])
 def test_rmsnorm_and_the_fused_joins(rt, dtype, T, H, eps, uo):
     k = rt.kernels(dtype)
     rng = np.random.default_rng(H)
@@ -706,10 +710,10 @@ def test_rmsnorm_and_the_fused_joins(rt, dtype, T, H, eps, uo):
     Hd2 = rt.upload(h)
     k.zk_norm_add_norm(ptr(up(rt, sub, dtype)), 0, None, 0.0, 0, Hd2.ptr, None, 0.0, 0, None, T, H, rt.stream)
     assert np.abs(rt.download(Hd2) - (h.astype(np.float64) + sub)).max() < 1e-6
-    # the sublayer's output as planes of partial sums (three; six for the wide rows, whose kernel
-    # takes them four a turn): the same bits as their sum in plane order, rounded to the
+    # the sublayer's output as planes of partial sums (three; six or eleven for the wide rows,
+    # whose kernels take them four or eight a turn): the same bits as their sum in plane order, rounded to the
     # activation type, gives when handed over as one tensor
-    P = 3 if H < 3000 else 6
+    P = 3 if H < 3000 else (11 if H == 4608 else 6)        # eleven: a second turn of eight
     planes = rng.normal(size=(P, T, H)).astype(np.float32)
     total = planes[0]
     for q in range(1, P):

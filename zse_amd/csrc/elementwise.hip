@@ -323,6 +323,114 @@ __global__ __launch_bounds__(256) void norm_add_norm_fast_kernel(
   }
 }
 
+// The same for the few rows of a decode step (up to 64 rows of 2,048 to 8,192 values): 1,024
+// threads a row instead of 256, so a thread holds one or two vectors (4 x 1024 x MAXV >= H) and can
+// ask for all planes of partial sums at once, eight a turn.  With so few rows the kernel's time is
+// its trips to memory and its two block sums, not its bytes: 8 rows of 4,608 values that come as
+// eight planes (27B shapes) 2.9 us less a launch, a decode step at batch 8 of 2B shapes 2.46 -> 2.42
+// ms, of 9B shapes (14 layers) 2.47 -> 2.40 ms, 2B shapes at batch 32 4.51 -> 4.40 ms; with 2,048
+// rows it loses (the 2B prefill 12.43 -> 12.75 ms), so more than 64 rows stay with the kernel
+// above.  The sums of the planes are the same bits; the two row sums are added up in another
+// order than by 256 threads, so which of the two kernels serves a launch depends on the rows and
+// the width alone, never on whether planes come.
+template <int MAXV>
+__global__ __launch_bounds__(1024) void norm_add_norm_wide_kernel(
+    const void* __restrict__ sub, int parts, const float* __restrict__ w_post, float eps_post, int uo_post,
+    float* __restrict__ h, const float* __restrict__ w_next, float eps_next, int uo_next,
+    act_t* __restrict__ out, int H) {
+  __shared__ float red[17];
+  const int r = blockIdx.x;
+  const act_t* s = (const act_t*)sub + (size_t)r * H;
+  const float* sf = (const float*)sub + (size_t)r * H;
+  const size_t plane = (size_t)gridDim.x * H;
+  float* hr = h + (size_t)r * H;
+  float v[MAXV][4], hv[MAXV][4], gp[MAXV][4], gn[MAXV][4];
+#pragma unroll
+  for (int j = 0; j < MAXV; j++) {
+    const int i = threadIdx.x * 4 + j * 4096;
+    if (i < H) {
+      if (parts <= 0) load4<act_t>(s + i, v[j]);
+      else load4<float>(sf + i, v[j]);
+      load4<float>(hr + i, hv[j]);
+      if (w_post) load4<float>(w_post + i, gp[j]);
+      if (w_next) load4<float>(w_next + i, gn[j]);
+    }
+  }
+  if (parts > 0) {
+    // a plane past the last is read from the last and not added; the planes are added in order
+    for (int p0 = 1; p0 < parts; p0 += 8) {
+      float t[MAXV][8][4];
+#pragma unroll
+      for (int j = 0; j < MAXV; j++) {
+        const int i = threadIdx.x * 4 + j * 4096;
+        if (i < H) {
+#pragma unroll
+          for (int q = 0; q < 8; q++) load4<float>(sf + (size_t)min(p0 + q, parts - 1) * plane + i, t[j][q]);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < MAXV; j++) {
+        if (threadIdx.x * 4 + j * 4096 < H) {
+#pragma unroll
+          for (int q = 0; q < 8; q++)
+            if (p0 + q < parts) {
+#pragma unroll
+              for (int e = 0; e < 4; e++) v[j][e] += t[j][q][e];
+            }
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < MAXV; j++)
+      if (threadIdx.x * 4 + j * 4096 < H) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[j][e] = to_f32(from_f32<act_t>(v[j][e]));
+      }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < MAXV; j++)
+    if (threadIdx.x * 4 + j * 4096 < H) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) ss += v[j][e] * v[j][e];
+    }
+  float rs = 1.f;
+  if (w_post) {
+    ss = block_sum(ss, red);
+    rs = rsqrtf(ss / (float)H + eps_post);
+  }
+  float ss2 = 0.f;
+#pragma unroll
+  for (int j = 0; j < MAXV; j++) {
+    const int i = threadIdx.x * 4 + j * 4096;
+    if (i < H) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        float t = v[j][e];
+        if (w_post) t = t * rs * (uo_post ? 1.f + gp[j][e] : gp[j][e]);
+        t = hv[j][e] + t;
+        v[j][e] = t;
+        ss2 += t * t;
+      }
+      store4(hr + i, v[j]);
+    }
+  }
+  if (!w_next) return;
+  ss2 = block_sum(ss2, red);
+  const float rs2 = rsqrtf(ss2 / (float)H + eps_next);
+  act_t* o = out + (size_t)r * H;
+#pragma unroll
+  for (int j = 0; j < MAXV; j++) {
+    const int i = threadIdx.x * 4 + j * 4096;
+    if (i < H) {
+      float y[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) y[e] = v[j][e] * rs2 * (uo_next ? 1.f + gn[j][e] : gn[j][e]);
+      store4(o + i, y);
+    }
+  }
+}
+
 // ------------------------------------------------------------------ gated activation
 
 __device__ __forceinline__ float gelu_tanh(float g) {
@@ -635,6 +743,19 @@ int zk_norm_add_norm(const void* sub, int sub_parts, const float* w_post, float 
   ZK_REQUIRE(T >= 0 && H > 0 && sub_parts >= 0, "zk_norm_add_norm: bad sizes");
   ZK_REQUIRE(w_next == nullptr || out != nullptr, "zk_norm_add_norm: next norm without output");
   if (T == 0) return 0;
+  if (ZSE_ACT_BF16 && T <= 64 && H % 4 == 0 && H >= 2048 && H <= 8192) {
+    // few rows of at least 2,048 values (see the kernel): a decode step's norms.  The 32-bit
+    // library keeps to one kernel whatever the rows, so that its results stay the same bits
+    // however a request's tokens are cut into steps.
+    hipStream_t st = (hipStream_t)stream;
+    if (H <= 4096)
+      norm_add_norm_wide_kernel<1><<<T, 1024, 0, st>>>(sub, sub_parts, w_post, eps_post, uo_post, h, w_next, eps_next,
+                                                       uo_next, (act_t*)out, H);
+    else
+      norm_add_norm_wide_kernel<2><<<T, 1024, 0, st>>>(sub, sub_parts, w_post, eps_post, uo_post, h, w_next, eps_next,
+                                                       uo_next, (act_t*)out, H);
+    return zk_launch_status("zk_norm_add_norm");
+  }
   if (H % 4 == 0 && H <= NF_MAXV * 1024) {
     hipStream_t st = (hipStream_t)stream;
 #define ZK_NAN_(V)                                                                                              \
