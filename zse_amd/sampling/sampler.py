@@ -153,6 +153,14 @@ class DeviceSampler:
         self.keep_from = rt.empty((max_rows,), F32)
         self.keep_ties = rt.empty((max_rows,), I32)
         self._pen = None                                    # (rows, tokens, scales) on the device, grown on demand
+        # the rows' temperatures, uniform numbers and cut-offs on their way to the device: page-locked,
+        # so their copies queue behind the step's kernels instead of waiting for them (``sample``
+        # reads its ids before it returns, so the next call finds the buffer free)
+        self._stage = rt.pinned(max_rows * 20)
+        self._stage_u = self._stage.array(0, max_rows, np.float64)
+        self._stage_t = self._stage.array(max_rows * 8, max_rows, np.float32)
+        self._stage_k = self._stage.array(max_rows * 12, max_rows, np.int32)
+        self._stage_p = self._stage.array(max_rows * 16, max_rows, np.float32)
 
     # ---- a run of steps without waiting for the host in between
     RING = 16       # results that may be on their way to the host at a time
@@ -227,16 +235,17 @@ class DeviceSampler:
         if any(greedy):
             k.zk_argmax(logits.ptr, self.ids.ptr, n, V, self.scratch.ptr, rt.stream)
         if not all(greedy):
-            t = np.array([1.0 if g else r["params"].temperature for r, g in zip(rows, greedy)], dtype=np.float32)
-            u = np.array([r["u"] for r in rows], dtype=np.float64)
-            rt.copy_h2d(self.temp.ptr, t)
-            rt.copy_h2d(self.u.ptr, u)
+            st = self._stage.ptr
+            self._stage_t[:n] = [1.0 if g else r["params"].temperature for r, g in zip(rows, greedy)]
+            self._stage_u[:n] = [r["u"] for r in rows]
+            rt.copy_h2d_async(self.temp.ptr, st + self.max_rows * 8, n * 4)
+            rt.copy_h2d_async(self.u.ptr, st, n * 8)
             cut = any(not g and (r["params"].top_k > 0 or r["params"].top_p < 1.0) for r, g in zip(rows, greedy))
             if cut:
-                rt.copy_h2d(self.top_k.ptr, np.array([0 if g else r["params"].top_k for r, g in zip(rows, greedy)],
-                                                     dtype=np.int32))
-                rt.copy_h2d(self.top_p.ptr, np.array([1.0 if g else r["params"].top_p for r, g in zip(rows, greedy)],
-                                                     dtype=np.float32))
+                self._stage_k[:n] = [0 if g else r["params"].top_k for r, g in zip(rows, greedy)]
+                self._stage_p[:n] = [1.0 if g else r["params"].top_p for r, g in zip(rows, greedy)]
+                rt.copy_h2d_async(self.top_k.ptr, st + self.max_rows * 12, n * 4)
+                rt.copy_h2d_async(self.top_p.ptr, st + self.max_rows * 16, n * 4)
                 self._cutoff(logits, n, V)
             k.zk_sample(logits.ptr, self.temp.ptr, self.u.ptr, self.keep_from.ptr if cut else None,
                         self.keep_ties.ptr if cut else None, self.ids2.ptr, n, V, self.scratch.ptr, rt.stream)
