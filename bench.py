@@ -15,8 +15,9 @@ two probe kernels reach on this very GPU (``frac_probed``).
 Before anything is timed the model is checked (``checked``): a two-layer slice of the very
 model that is timed (same seed, so the same tensors) runs whole prompts, portions and single
 tokens in 32-bit and in bfloat16 against the plain implementation under ``tests/plain`` on the
-same weights made on the host, and the full model's decode steps through captured graphs must
-pick the same tokens as eager steps.  A failed check ends the run with an error.
+same weights made on the host, and at every batch size that is timed the full model's decode
+steps through the timed path (captured graphs or launch lists, ids fed on the device) must pick
+the same tokens as steps launched call by call.  A failed check ends the run with an error.
 
 ``--workload`` runs one of the two larger workloads through ``Engine.generate`` instead, end to
 end: 9b = 32 requests with prompts of 128 to 4,096 tokens, 256 greedy tokens each, portions of
@@ -173,23 +174,47 @@ def check_slice(cfg, rt, seed, std, gain_std):
     return out
 
 
-def check_graphs(model, rt, vocab):
-    """The model that is timed: tokens picked through captured decode steps equal those of eager steps."""
+def check_decode_path(model, rt, vocab, B, use_graphs):
+    """The model that is timed, at a batch size that is timed: the ids that come out of the
+    timed path (graphs up to 16 requests, launch lists above, ids picked on the device and fed
+    to the next step from there) equal those of steps launched call by call from Python whose
+    logits the host reads."""
     from zse_amd.engine.runner import StepEntry, StepRunner
-    rng = np.random.default_rng(5)
-    prompts = [rng.integers(0, vocab, 24 + 3 * i).tolist() for i in range(8)]
+    from zse_amd.sampling.sampler import DeviceSampler, SamplingParams
+    rng = np.random.default_rng(5 + B)
+    prompts = [rng.integers(0, vocab, 24 + 3 * (i % 11)).tolist() for i in range(B)]
+    n_steps = 7
     picked = []
-    for graphs in (False, True):
-        runner = StepRunner(model, rt, "bfloat16", page_size=16, cache_tokens=1024, max_seqs=8, max_batch_tokens=512,
-                            max_model_len=4096, use_graphs=graphs)
-        z = runner.step([StepEntry(i, p, [len(p) - 1]) for i, p in enumerate(prompts)])
-        ids = [z.argmax(axis=1).tolist()]
-        for _ in range(6):
-            z = runner.step([StepEntry(i, [t], [0]) for i, t in enumerate(ids[-1])])
-            ids.append(z.argmax(axis=1).tolist())
-        if graphs and not any(isinstance(g, int) for g in runner.graphs.values()):
-            raise SystemExit("bench.py: no decode step was captured into a graph")
+    for timed in (False, True):
+        runner = StepRunner(model, rt, "bfloat16", page_size=16, cache_tokens=B * 96, max_seqs=B,
+                            max_batch_tokens=max(2048, B), max_model_len=4096, use_graphs=timed and use_graphs,
+                            use_steplists=timed)
+        ids = []
+        for at in range(0, B, 16):                 # the prompts, sixteen a step
+            z = runner.step([StepEntry(i, prompts[i], [len(prompts[i]) - 1]) for i in range(at, min(at + 16, B))])
+            ids += z.argmax(axis=1).tolist()
+        ids = [ids]
+        if not timed:
+            for _ in range(n_steps):
+                z = runner.step([StepEntry(i, [t], [0]) for i, t in enumerate(ids[-1])])
+                ids.append(z.argmax(axis=1).tolist())
+        else:
+            sampler = DeviceSampler(rt, runner.k, B)
+            sampler.prepare_run([{"params": SamplingParams(temperature=0.0), "u": 0.0} for _ in range(B)], [[0.0] * B])
+            fed, pending = None, []
+            for _ in range(n_steps):
+                toks = ids[0] if fed is None else [0] * B
+                logits = runner.step([StepEntry(i, [t], [0]) for i, t in enumerate(toks)], download=False,
+                                     tokens_from=fed)
+                pending.append(sampler.sample_deferred(logits, 0))
+                fed = pending[-1].device_ptr
+            ids += [list(p.result()) for p in pending]
+            if use_graphs and B <= runner.graph_max_batch and not any(isinstance(g, int) for g in runner.graphs.values()):
+                raise SystemExit("bench.py: no decode step was captured into a graph")
+            if B > runner.graph_max_batch and runner.steplist_runs == 0:
+                raise SystemExit("bench.py: no decode step ran from its launch list")
         picked.append(ids)
+        runner.close()
         del runner
     return picked[0] == picked[1]
 
@@ -317,22 +342,23 @@ def main():
     t0 = time.time()
     model = random_model(cfg, "bfloat16", seed=SEED, std=STD, gain_std=GAIN_STD, rt=rt)
     V = cfg["vocab_size"]
+    points = sorted({int(x) for x in a.points.split(",") if x} | {a.batch})
     check = None
     if not a.no_check and not a.only:
         errs = check_slice(cfg, rt, SEED, STD, GAIN_STD)
-        same_ids = check_graphs(model, rt, V)
+        same_ids = all(check_decode_path(model, rt, V, B, not a.no_graphs) for B in points)
         # 32-bit: summation order only (2e-5 of the largest logit seen at these widths);
         # bfloat16: inputs of every product rounded to 8 bits (under 1 % seen)
         ok = errs["float32"] < 1e-4 and errs["bfloat16"] < 0.02 and same_ids
         check = {"fp32_max_rel_err": float(f"{errs['float32']:.3g}"), "bf16_max_rel_err": float(f"{errs['bfloat16']:.3g}"),
-                 "graph_ids_equal_eager": bool(same_ids), "slice_layers": 2, "cuts": "whole, portions, token by token, mixed"}
+                 "timed_path_ids_equal_eager": bool(same_ids), "at_batches": points, "slice_layers": 2,
+                 "cuts": "whole, portions, token by token, mixed"}
         log(f"check: {check} ({time.time() - t0:.1f} s)")
         if not ok:
             raise SystemExit(f"bench.py: the engine does not agree with the plain implementation: {check}")
     peak_bw, peak_fl = probe_peaks(rt)
     log(f"probes: {peak_bw / 1e9:.0f} GB/s streamed, {peak_fl / 1e12:.0f} TFLOP/s bf16 on the matrix cores")
 
-    points = sorted({int(x) for x in a.points.split(",") if x} | {a.batch})
     max_b = max(points)
     page = 16
     longest = max(a.context, a.prefill_tokens)       # a prompt longer than the decode context still fits
@@ -439,7 +465,7 @@ def main():
                    "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
                    "sliding_window": cfg["sliding_window"], "global_batch": a.batch, "seq_len": a.context,
                    "prompt_len": a.prefill_tokens, "page_size": page, "parallelism": "single-gpu",
-                   "graphs": int(runner.use_graphs)},
+                   "graphs": int(runner.use_graphs), "graph_max_batch": runner.graph_max_batch},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(byts / step_s / 1e9, 1), "peak": PEAK_HBM / 1e9,
                      "unit": "GB/s", "frac": round(byts / step_s / PEAK_HBM, 4),

@@ -106,10 +106,12 @@ def chunked_steps(streams, sizes=(7, 2, 5, 3, 2, 11, 2, 4)):
     return steps
 
 
-def mixed_steps(streams, seed=0, max_live=4, decode_tail=12, chunk_choices=(2, 3, 5, 9), room=None, page=1):
+def mixed_steps(streams, seed=0, max_live=4, decode_tail=12, chunk_choices=(2, 3, 5, 9), room=None, page=1,
+                skip=0.15):
     """Up to ``max_live`` requests at a time: prompt portions of some beside single
     tokens of others (a request decodes one by one over its last ``decode_tail``
-    tokens); requests enter as others leave; some sit a step out.  ``room``: pages of
+    tokens, or ``decode_tail[request]`` where a mapping is given); requests enter as others leave; some sit a step out (each with probability
+    ``skip``).  ``room``: pages of
     ``page`` tokens the pool has; a request enters only while the live requests, each at
     its full length, and it fit together."""
     rng = np.random.default_rng(seed)
@@ -126,10 +128,11 @@ def mixed_steps(streams, seed=0, max_live=4, decode_tail=12, chunk_choices=(2, 3
             fed[r] = 0
         entries, ends = [], []
         for r in list(live):
-            if len(live) > 1 and rng.random() < 0.15:
+            if len(live) > 1 and rng.random() < skip:
                 continue                                  # left out of this step
             left = len(streams[r]) - fed[r]
-            n = 1 if left <= decode_tail else min(int(rng.choice(chunk_choices)), left - decode_tail)
+            tail = decode_tail[r] if isinstance(decode_tail, dict) else decode_tail
+            n = 1 if left <= tail else min(int(rng.choice(chunk_choices)), left - tail)
             entries.append((r, n))
             fed[r] += n
             if fed[r] == len(streams[r]):
