@@ -189,3 +189,36 @@ def test_attention_workspace_follows_the_models_limits():
     # a context the decode kernel cannot join is refused when the runner is made, with the numbers
     with pytest.raises(ValueError, match="longest context"):
         part.prepare(k, "bfloat16", 64, 300000, 16)
+
+
+def test_a_pool_whose_ids_begin_at_one_and_the_page_a_step_begins_to_fill():
+    from zse_amd.cache.manager import CacheManager, GroupInfo
+    from zse_amd.cache.pages import PagePool
+    pool = PagePool(3, first_id=1)
+    got = [pool.alloc("a") for _ in range(3)]
+    assert got == [1, 2, 3] and pool.free_pages == 0
+    with pytest.raises(ValueError):
+        pool.free(0, "a")
+    pool.free(2, "a")
+    pool.check()
+    assert pool.alloc("b") == 2
+
+    m = CacheManager([GroupInfo(8, [0], 6), GroupInfo(None, [1], 6)], page_size=4, max_seqs=2, max_model_len=24,
+                     first_page=1)
+    m.add("r")
+    assert m.reserve("r", 6)
+    # 6 tokens: page 0 of the request is filled, its page 1 is begun and was never written
+    assert m.untouched_page("r", 0, 6) == m.table("r", 0)[1] and m.untouched_page("r", 1, 6) == m.table("r", 1)[1]
+    assert min(m.table("r", 0)) >= 1
+    m.commit("r", 6)
+    assert m.reserve("r", 7)
+    assert m.untouched_page("r", 0, 7) is None          # the request wrote to that page in the step before
+    m.commit("r", 7)
+    assert m.reserve("r", 8) and m.untouched_page("r", 0, 8) is None      # a step that fills its last page
+    m.commit("r", 8)
+    assert m.reserve("r", 9)
+    assert m.untouched_page("r", 0, 9) == m.table("r", 0)[2]
+    m.commit("r", 9)
+    # a step of many tokens: only the page it ends in can be left half filled
+    assert m.reserve("r", 22) and m.untouched_page("r", 1, 22) == m.table("r", 1)[5]
+    m.check()

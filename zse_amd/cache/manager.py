@@ -61,12 +61,14 @@ def group_needs(needs: Sequence[object]) -> List[GroupInfo]:
 
 class CacheManager:
     def __init__(self, groups: Sequence[GroupInfo], page_size: int, max_seqs: int,
-                 max_model_len: int, slot_bytes: int = 0):
+                 max_model_len: int, slot_bytes: int = 0, first_page: int = 0):
         if page_size <= 0:
             raise ValueError("page_size must be positive")
         self.page_size = int(page_size)
         self.groups = list(groups)
-        self.pools = [PagePool(g.num_pages) for g in self.groups]
+        # first_page = 1: the owner of the slabs keeps page 0 of every slab to itself (cleared,
+        # never handed out), which is what a kernel reads for a table entry without a page
+        self.pools = [PagePool(g.num_pages, first_page) for g in self.groups]
         self.slots = StateSlots(max_seqs, slot_bytes)
         self.max_model_len = int(max_model_len)
         self.max_blocks = -(-self.max_model_len // self.page_size)
@@ -160,6 +162,21 @@ class CacheManager:
         self.slots.release(req)
 
     # ---- what a step needs
+    def untouched_page(self, req, group: int, upto: int) -> Optional[int]:
+        """The page that a step bringing the request to ``upto`` tokens begins to fill without
+        filling it: its id, if the request has not written to it before (it then still holds
+        what its last owner left), else None.  Pages are filled in the order of positions, so
+        a page is untouched exactly when all its positions lie at or behind the computed
+        length; a step fills every such page but, at most, the last."""
+        if upto % self.page_size == 0:
+            return None
+        r = self._reqs[req]
+        j = (upto - 1) // self.page_size
+        if j * self.page_size < r.computed:
+            return None
+        page = r.tables[group][j]
+        return page if page >= 0 else None
+
     def table(self, req, group: int) -> List[int]:
         return self._reqs[req].tables[group]
 

@@ -16,12 +16,19 @@ class OutOfPages(RuntimeError):
 
 
 class PagePool:
-    def __init__(self, num_pages: int):
+    def __init__(self, num_pages: int, first_id: int = 0):
+        """``num_pages`` pages with the ids ``first_id`` .. ``first_id + num_pages - 1``.  An owner
+        of the pages' memory that keeps a page of its own in front of them (one that is never
+        handed out, for table entries that name no page) starts the ids at 1."""
         if num_pages <= 0:
             raise ValueError(f"a pool needs at least one page, got {num_pages}")
+        if first_id < 0:
+            raise ValueError("page ids are not negative")
         self.num_pages = int(num_pages)
-        self._free: List[int] = list(range(self.num_pages - 1, -1, -1))   # pop() gives 0 first
-        self._owner: List[Optional[object]] = [None] * self.num_pages
+        self.first_id = int(first_id)
+        last = self.first_id + self.num_pages - 1
+        self._free: List[int] = list(range(last, self.first_id - 1, -1))   # pop() gives the first id first
+        self._owner: List[Optional[object]] = [None] * (last + 1)
 
     @property
     def free_pages(self) -> int:
@@ -42,7 +49,7 @@ class PagePool:
         return p
 
     def free(self, page: int, owner) -> None:
-        if not (0 <= page < self.num_pages):
+        if not (self.first_id <= page < self.first_id + self.num_pages):
             raise ValueError(f"page {page} is not in the pool")
         if self._owner[page] is None:
             raise RuntimeError(f"page {page} freed twice")
@@ -59,6 +66,6 @@ class PagePool:
         free = set(self._free)
         if len(free) != len(self._free):
             raise AssertionError("a page is on the free list twice")
-        for p in range(self.num_pages):
+        for p in range(self.first_id, self.first_id + self.num_pages):
             if (p in free) == (self._owner[p] is not None):
                 raise AssertionError(f"page {p}: free={p in free}, owner={self._owner[p]!r}")

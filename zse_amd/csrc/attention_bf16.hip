@@ -517,8 +517,10 @@ __global__ __launch_bounds__(NW * 64, (HD16 <= 8 && NW <= 4) ? 2 : 1) void attn_
   struct Pages { int k[PPT], v[PPT]; };
   struct Stage { bf16x8 k[PPT], v[PPT]; };
   // A key past the request's last (in its last tile, or in the tile fetched after the last) is
-  // read from wherever its table entry points, page 0 where there is none: it is masked, and
-  // the cache holds finite values everywhere.
+  // read from wherever its table entry points, page 0 where there is none.  It is masked, but
+  // its value still meets a weight of 0 in the second product, and 0 x NaN is NaN: the caller
+  // keeps page 0 cleared and clears a page before a request first writes to part of it, so
+  // what is read here is the request's own or zero, never what another request left.
   auto look_up = [&](int key0, Pages& pg) {
     const int first = key0 >> bsh;
 #pragma unroll
@@ -757,7 +759,9 @@ __global__ __launch_bounds__(256, 2) void attn_decode_kernel(AttnParams p) {
   const int hd = p.hd, bsh = p.bs_shift, bmask = p.bs - 1, nkv = p.nkv;
   // The pages of the chunk's (up to two) tiles are asked for before the request's length is
   // known, beside it: where a key lies follows from the chunk alone.  A key past the context is
-  // masked below, so any page serves for it (a hole in the table reads page 0).
+  // masked below; a hole in the table reads page 0, which the caller keeps cleared, and the
+  // places of a request's last page behind its last token are cleared too (a masked value
+  // still meets a weight of 0 in the second product, and 0 x NaN is NaN).
   int kpage[2][2], vpage[2][2];
 #pragma unroll
   for (int i = 0; i < 2; i++) {

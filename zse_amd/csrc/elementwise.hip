@@ -9,6 +9,8 @@
 // of K and V into pages :961-1012.
 #include "common.h"
 
+#include <algorithm>
+
 thread_local std::string zk_error;
 int zk_fail(const char* msg) {
   zk_error = msg;
@@ -699,6 +701,23 @@ __global__ void zero_kernel(uint32_t* __restrict__ p, size_t n_words) {
   if (i < n_words) p[i] = 0u;
 }
 
+// Clears whole pages in several slabs at once: block (x, y) clears page pages.id[x] of slab y.
+// A slab is an array of pages of slab_page_bytes[y] bytes each (a multiple of 16), so a page id
+// names the same place in each of them.  The ids come by value with the launch.
+#define ZERO_PAGES_MOST 64
+struct PageIds {
+  int n;
+  int id[ZERO_PAGES_MOST];
+};
+__global__ __launch_bounds__(256) void zero_pages_kernel(void* const* __restrict__ slabs,
+                                                         const unsigned long long* __restrict__ slab_page_bytes,
+                                                         PageIds pages) {
+  const unsigned long long nbytes = slab_page_bytes[blockIdx.y];
+  uint4* dst = (uint4*)((char*)slabs[blockIdx.y] + (size_t)pages.id[blockIdx.x] * nbytes);
+  const uint4 z = make_uint4(0u, 0u, 0u, 0u);
+  for (size_t i = threadIdx.x; i < nbytes / 16; i += 256) dst[i] = z;
+}
+
 // ------------------------------------------------------------------ C interface
 
 extern "C" {
@@ -850,6 +869,26 @@ int zk_zero(void* p, size_t nbytes, void* stream) {
   ZK_REQUIRE((n + 255) / 256 < 2147483647ull, "zk_zero: too many bytes");
   zero_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>((uint32_t*)p, n);
   return zk_launch_status("zk_zero");
+}
+
+// Clears pages ``pages[0 .. n_pages)`` (host array of ids) of each of ``n_slabs`` slabs, whose
+// base addresses and page sizes in bytes lie in device memory.  Launched per 64 ids.
+int zk_zero_pages(const void* slabs, const void* slab_page_bytes, int n_slabs, const int* pages, int n_pages,
+                  void* stream) {
+  ZK_REQUIRE(n_slabs >= 0 && n_slabs <= 65535 && n_pages >= 0, "zk_zero_pages: bad counts");
+  if (n_slabs == 0 || n_pages == 0) return 0;
+  ZK_REQUIRE(slabs != nullptr && slab_page_bytes != nullptr && pages != nullptr, "zk_zero_pages: null argument");
+  for (int at = 0; at < n_pages; at += ZERO_PAGES_MOST) {
+    PageIds ids;
+    ids.n = std::min(ZERO_PAGES_MOST, n_pages - at);
+    for (int i = 0; i < ids.n; i++) {
+      ZK_REQUIRE(pages[at + i] >= 0, "zk_zero_pages: negative page id");
+      ids.id[i] = pages[at + i];
+    }
+    zero_pages_kernel<<<dim3(ids.n, n_slabs), 256, 0, (hipStream_t)stream>>>(
+        (void* const*)slabs, (const unsigned long long*)slab_page_bytes, ids);
+  }
+  return zk_launch_status("zk_zero_pages");
 }
 
 }  // extern "C"

@@ -16,6 +16,7 @@ HIP graph per batch size as there (model_runner.py:1806-1932).
 """
 from __future__ import annotations
 
+import ctypes
 import inspect
 
 import weakref
@@ -180,7 +181,9 @@ class StepRunner:
             cc = CallCache(need=need)
             if isinstance(need, PagedKV):
                 cc.group = gid_of[i]
-                pages = groups[cc.group].num_pages
+                # page 0 of every slab is the runner's own: cleared here, never handed out and
+                # never written, it is what kernels read where a table names no page
+                pages = groups[cc.group].num_pages + 1
                 shape = (pages, need.num_kv_heads, self.page_size, need.head_dim)
                 cc.k = rt.zeros(shape, self.dtype)
                 mixer = model.blocks[model.plan.order[i].layer].mixer
@@ -195,7 +198,16 @@ class StepRunner:
                 slot_bytes += (int(need.nbytes) + 15) // 16 * 16
             self.caches.append(cc)
         self.slot_bytes = slot_bytes
-        self.manager = CacheManager(groups, self.page_size, self.max_seqs, self.max_model_len, slot_bytes)
+        self.manager = CacheManager(groups, self.page_size, self.max_seqs, self.max_model_len, slot_bytes,
+                                    first_page=1)
+        # per group: the base addresses and page sizes of its layers' slabs, for the kernel that
+        # clears a page in all of them
+        self._slabs = []
+        for gid in range(len(groups)):
+            ts = [t for cc in self.caches if cc.group == gid and cc.k is not None for t in (cc.k, cc.v)]
+            ptrs = rt.upload(np.array([t.ptr for t in ts], dtype=np.uint64).view(np.float64), "float64")
+            sizes = rt.upload(np.array([t.nbytes // t.shape[0] for t in ts], dtype=np.uint64).view(np.float64), "float64")
+            self._slabs.append((ptrs, sizes, len(ts)))
         self.state = rt.zeros((self.max_seqs, max(slot_bytes // 4, 1)), F32) if slot_bytes else None
         # the manager tells us of every admission; a weak reference, so that runner and manager
         # do not hold each other (a runner dropped by its owner frees its memory at once)
@@ -262,6 +274,25 @@ class StepRunner:
 
     def add(self, req) -> int:
         return self.manager.add(req)
+
+    def _clear_untouched(self, entries) -> None:
+        """A page that a request begins to fill in this step without filling it still holds, in
+        the places behind the request's last token, what the page's last owner left there.  The
+        attention kernels read whole tiles of keys and values and mask afterwards; a masked
+        value takes part in a matrix product with weight 0, and 0 x NaN is NaN.  So such a page is
+        cleared before the step writes to it: whatever a request's table names then holds the
+        request's own values or zeros, and nothing another request computed can reach it."""
+        m = self.manager
+        for g in range(len(m.groups)):
+            pages = []
+            for e in entries:
+                p = m.untouched_page(e.req, g, m.computed(e.req) + len(e.tokens))
+                if p is not None:
+                    pages.append(p)
+            if pages:
+                ptrs, sizes, n = self._slabs[g]
+                arr = (ctypes.c_int * len(pages))(*pages)
+                self.k.zk_zero_pages(ptrs.ptr, sizes.ptr, n, arr, len(pages), self.rt.stream)
 
     def finish(self, req) -> None:
         self.manager.release(req)
@@ -513,6 +544,7 @@ class StepRunner:
                                  f"cannot give them: {m.stats()}")
         if tokens_from is not None and T != R:
             raise ValueError("tokens_from serves steps in which every request brings one token")
+        self._clear_untouched(entries)
         self.rt.wait_event(self.meta_copied)     # the last step's copy has left the host buffer
         bucket = self._graph_bucket(entries)
         if bucket:
