@@ -215,6 +215,81 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(rt):
         assert not runner.graph_safe          # the toy reads the step's description on the host
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_part_brings_a_kernel_of_its_own(rt, dtype):
+    """The toy mixer's recurrence as a kernel in a file beside the tests, registered with one
+    call: the framework compiles it, calls it like its own, repeats it from launch lists and
+    replays it inside captured graphs, and no file of the framework names it.  Same weights,
+    same tokens: the bits of the toy mixer whose recurrence runs on the host."""
+    import os
+    import subprocess
+    from conftest import ROOT
+    from zse_amd.config import BlockSpec, EmbeddingSpec, GatedMLPSpec, HeadSpec, LayerCall, ModelPlan, NormSpec
+    from zse_amd.config import Architecture, register_architecture, unregister_architecture
+    from zse_amd.engine.loading import random_model
+    from zse_amd.engine.runner import StepEntry, StepRunner
+    from toy_state import DecaySpec, toy_architecture
+    from toy_decay_device import DeviceDecaySpec
+
+    H, V, I, L, A = 64, 200, 96, 2, 0.75
+
+    def plan_with(spec, name):
+        def plan_of(cfg):
+            norm = lambda n: NormSpec(H, 1e-6, False, n)
+            layers = tuple(BlockSpec("prenorm", spec(H, A, f"l{l}.mix.w"),
+                                     GatedMLPSpec(H, I, "silu", {r: f"l{l}.ffn.{r}" for r in ("gate", "up", "down")}),
+                                     {"pre_mixer": norm(f"l{l}.n1"), "pre_ffn": norm(f"l{l}.n2")}) for l in range(L))
+            return ModelPlan(name, H, V, 512, EmbeddingSpec(V, H, 1.0, "emb"), layers,
+                             tuple(LayerCall(l) for l in range(L)), norm("final"), HeadSpec(V, H, None, "emb"))
+        return plan_of
+
+    rng = np.random.default_rng(0)
+    streams = {"a": rng.integers(0, V, 29).tolist(), "b": rng.integers(0, V, 17).tolist()}
+    # portions of sizes that come back, then single tokens side by side: shapes repeat, so launch
+    # lists run and the graph of bucket 2 is captured and replayed
+    steps = [[("a", 5)], [("b", 5)], [("a", 5), ("b", 3)], [("a", 5), ("b", 3)], [("a", 2)], [("b", 2)]]
+    steps += [[("a", 1), ("b", 1)] for _ in range(4)] + [[("a", 1)] for _ in range(8)]
+
+    def run(runner):
+        fed = {r: 0 for r in streams}
+        rows = {r: [] for r in streams}
+        for st in steps:
+            z = runner.step([StepEntry(r, streams[r][fed[r]:fed[r] + n], [n - 1]) for r, n in st])
+            for (r, n), row in zip(st, z):
+                rows[r].append(row.copy())
+                fed[r] += n
+        assert all(fed[r] == len(t) for r, t in streams.items())
+        return {r: np.stack(v) for r, v in rows.items()}
+
+    limits = dict(page_size=4, cache_tokens=64, max_seqs=3, max_batch_tokens=64, max_model_len=128)
+    with toy_architecture("ToyDecayLM", plan_with(DecaySpec, "ToyDecayLM")):
+        host_model = random_model({"architectures": ["ToyDecayLM"]}, dtype, seed=4, std=0.1, gain_std=0.1, rt=rt)
+        want = run(StepRunner(host_model, rt, dtype, use_graphs=False, **limits))
+    register_architecture(Architecture("ToyDecayDeviceLM", lambda d: d, plan_with(DeviceDecaySpec, "ToyDecayDeviceLM")))
+    try:
+        model = random_model({"architectures": ["ToyDecayDeviceLM"]}, dtype, seed=4, std=0.1, gain_std=0.1, rt=rt)
+        plain = StepRunner(model, rt, dtype, use_graphs=False, use_steplists=False, **limits)
+        assert plain.graph_safe and hasattr(plain.k, "zk_toy_decay")
+        got_plain = run(plain)
+        runner = StepRunner(model, rt, dtype, use_graphs=True, **limits)
+        got = run(runner)
+        assert runner.use_steplists and runner.steplist_runs >= 2, "the part's kernel kept steps from being written down"
+        assert any(isinstance(g, int) for g in runner.graphs.values()), "no decode step was captured"
+        names = {runner.k._dll.zk_steplist_name(h, i).decode() for h in runner.steplists.values()
+                 for i in range(runner.k.steplist_size(h))}
+        assert "zk_toy_decay" in names
+        runner.close(), plain.close()
+    finally:
+        unregister_architecture("ToyDecayDeviceLM")
+    for r in streams:
+        assert np.array_equal(got[r], got_plain[r]), f"{r}: lists and graphs against launches from Python"
+        assert np.array_equal(got[r], want[r]), f"{r}: the kernel against the recurrence on the host"
+    # nothing under zse_amd/ knows the toy
+    hits = subprocess.run(["grep", "-rl", "toy_decay", os.path.join(ROOT, "zse_amd"), "--include=*.py",
+                           "--include=*.hip", "--include=*.h", "--include=*.cpp"], capture_output=True, text=True)
+    assert hits.stdout.strip() == "", hits.stdout
+
+
 def test_toy_mixer_with_state_through_the_engine(rt):
     """The same toy mixer behind the scheduler: layer 0 keeps its recurrence in the request's
     state slot, layer 1 is the framework's attention over pages.  Six requests share two slots

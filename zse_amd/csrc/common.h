@@ -76,3 +76,24 @@ int zk_launch_status(const char* what);
   do {                        \
     if (!(cond)) return zk_fail(msg); \
   } while (0)
+
+// The definitions behind the three declarations above and the two functions through which a
+// caller asks a library for its last message and its storage type.  Each shared library has
+// them once: the kernel libraries in elementwise.hip, a library of a part's own kernels in its
+// own source file.
+#define ZK_DEFINE_HOST_SIDE                                               \
+  thread_local std::string zk_error;                                      \
+  int zk_fail(const char* msg) {                                          \
+    zk_error = msg;                                                       \
+    return -1;                                                            \
+  }                                                                       \
+  int zk_launch_status(const char* what) {                                \
+    hipError_t e = hipGetLastError();                                     \
+    if (e != hipSuccess) {                                                \
+      zk_error = std::string(what) + ": " + hipGetErrorString(e);         \
+      return (int)e;                                                      \
+    }                                                                     \
+    return 0;                                                             \
+  }                                                                       \
+  extern "C" const char* zk_last_error() { return zk_error.c_str(); }     \
+  extern "C" int zk_act_is_bf16() { return ZSE_ACT_BF16; }

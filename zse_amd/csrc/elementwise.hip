@@ -11,19 +11,7 @@
 
 #include <algorithm>
 
-thread_local std::string zk_error;
-int zk_fail(const char* msg) {
-  zk_error = msg;
-  return -1;
-}
-int zk_launch_status(const char* what) {
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    zk_error = std::string(what) + ": " + hipGetErrorString(e);
-    return (int)e;
-  }
-  return 0;
-}
+ZK_DEFINE_HOST_SIDE
 
 // ------------------------------------------------------------------ embedding
 
@@ -721,9 +709,6 @@ __global__ __launch_bounds__(256) void zero_pages_kernel(void* const* __restrict
 // ------------------------------------------------------------------ C interface
 
 extern "C" {
-
-const char* zk_last_error() { return zk_error.c_str(); }
-int zk_act_is_bf16() { return ZSE_ACT_BF16; }
 
 int zk_embed(const void* table, const int* tokens, float* out, float scale, int T, int H, int V,
              int strip, void* stream) {

@@ -10,9 +10,17 @@
 // sequence from C++.  The reference drives each launch from Python (it measured about 7 us a
 // launch, orchestrator/hip_graph.py:3-5) and has a C dispatch table for single launches that
 // is switched off (orchestrator/fast_dispatch.py:151-337).
+//
+// The entry points are a table, not a list of names known here: a row holds a name, the
+// number of arguments and a function that calls the entry point from its arguments as words
+// (packed_call.h).  This library's own entry points enter the table when it is loaded; a
+// library of a part's own kernels adds its rows with zk_steplist_register.
 #include "common.h"
+#include "packed_call.h"
 
 #include <cstring>
+#include <mutex>
+#include <string>
 #include <vector>
 
 extern "C" {
@@ -49,105 +57,95 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
 
 namespace {
 
-// One written-down call: which entry point, and its arguments as 64-bit words in the order
-// of the C signature (a pointer or size as it is, an int sign-extended, a float as its bits).
-// The last argument of every entry point is the stream; a run puts its own there.
+constexpr int MOST_ARGS = 24;
+
+// One written-down call: a row of the table, and the entry point's arguments as 64-bit words
+// in the order of its C signature.  The last argument of every entry point is the stream; a
+// run puts its own there.
 struct StepCall {
   int op;
-  int n;
-  uint64_t a[24];
+  uint64_t a[MOST_ARGS];
 };
 
 struct StepList {
   std::vector<StepCall> calls;
 };
 
-inline void* P(uint64_t w) { return (void*)(uintptr_t)w; }
-inline int I(uint64_t w) { return (int)(int64_t)w; }
-inline size_t Z(uint64_t w) { return (size_t)w; }
-inline float F(uint64_t w) {
-  const uint32_t b = (uint32_t)w;
-  float f;
-  memcpy(&f, &b, 4);
-  return f;
-}
-
-struct OpInfo {
-  const char* name;
+struct Op {
+  std::string name;
   int nargs;
+  zk_packed_fn fn;
 };
 
-enum {
-  OP_EMBED, OP_RMSNORM, OP_NORM_ADD_NORM, OP_GATED_ACT, OP_SOFTCAP, OP_ROPE_CACHE_WRITE, OP_ZERO, OP_GEMM_PLAIN,
-  OP_ATTENTION_PLAIN, OP_GEMM_BF16, OP_QKV_ROPE_BF16, OP_ATTENTION_BF16, OP_COUNT
-};
+std::mutex table_lock;
 
-const OpInfo OPS[OP_COUNT] = {
-    {"zk_embed", 9},        {"zk_rmsnorm", 10},   {"zk_norm_add_norm", 13},    {"zk_gated_act", 6},
-    {"zk_softcap", 4},      {"zk_rope_cache_write", 14}, {"zk_zero", 3},        {"zk_gemm_plain", 10},
-    {"zk_attention_plain", 19}, {"zk_gemm_bf16", 16}, {"zk_qkv_rope_bf16", 19}, {"zk_attention_bf16", 24},
-};
+// Room for every row is set aside once, so a row never moves: a list may be launched (rows
+// read without the lock) while another thread adds a row.
+constexpr size_t MOST_OPS = 1024;
 
-int run_call(const StepCall& c, void* s) {
-  const uint64_t* a = c.a;
-  switch (c.op) {
-    case OP_EMBED:
-      return zk_embed(P(a[0]), (const int*)P(a[1]), (float*)P(a[2]), F(a[3]), I(a[4]), I(a[5]), I(a[6]), I(a[7]), s);
-    case OP_RMSNORM:
-      return zk_rmsnorm(P(a[0]), I(a[1]), (const int*)P(a[2]), (const float*)P(a[3]), P(a[4]), F(a[5]), I(a[6]),
-                        I(a[7]), I(a[8]), s);
-    case OP_NORM_ADD_NORM:
-      return zk_norm_add_norm(P(a[0]), I(a[1]), (const float*)P(a[2]), F(a[3]), I(a[4]), (float*)P(a[5]),
-                              (const float*)P(a[6]), F(a[7]), I(a[8]), P(a[9]), I(a[10]), I(a[11]), s);
-    case OP_GATED_ACT:
-      return zk_gated_act(P(a[0]), P(a[1]), I(a[2]), I(a[3]), I(a[4]), s);
-    case OP_SOFTCAP:
-      return zk_softcap((float*)P(a[0]), Z(a[1]), F(a[2]), s);
-    case OP_ROPE_CACHE_WRITE:
-      return zk_rope_cache_write(P(a[0]), (const int*)P(a[1]), (const int*)P(a[2]), (const float*)P(a[3]), I(a[4]),
-                                 P(a[5]), P(a[6]), I(a[7]), I(a[8]), I(a[9]), I(a[10]), I(a[11]), I(a[12]), s);
-    case OP_ZERO:
-      return zk_zero(P(a[0]), Z(a[1]), s);
-    case OP_GEMM_PLAIN:
-      return zk_gemm_plain(P(a[0]), I(a[1]), P(a[2]), P(a[3]), I(a[4]), I(a[5]), I(a[6]), I(a[7]), I(a[8]), s);
-    case OP_ATTENTION_PLAIN:
-      return zk_attention_plain(P(a[0]), I(a[1]), P(a[2]), P(a[3]), (const int*)P(a[4]), I(a[5]), (const int*)P(a[6]),
-                                (const int*)P(a[7]), P(a[8]), I(a[9]), I(a[10]), I(a[11]), I(a[12]), I(a[13]),
-                                F(a[14]), F(a[15]), I(a[16]), I(a[17]), s);
-#if ZSE_ACT_BF16
-    case OP_GEMM_BF16: {
-      // the number of partial-sum planes follows from the shape: the Python side read it when
-      // the call was written down and laid the next call out accordingly; here it is dropped
-      int parts = 0;
-      return zk_gemm_bf16(P(a[0]), I(a[1]), P(a[2]), P(a[3]), I(a[4]), I(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]),
-                          F(a[10]), I(a[11]), P(a[12]), Z(a[13]), a[14] ? &parts : nullptr, s);
-    }
-    case OP_QKV_ROPE_BF16:
-      return zk_qkv_rope_bf16(P(a[0]), I(a[1]), P(a[2]), P(a[3]), I(a[4]), I(a[5]), I(a[6]), I(a[7]),
-                              (const int*)P(a[8]), (const int*)P(a[9]), (const float*)P(a[10]), P(a[11]), P(a[12]),
-                              I(a[13]), I(a[14]), I(a[15]), I(a[16]), I(a[17]), s);
-    case OP_ATTENTION_BF16:
-      return zk_attention_bf16(P(a[0]), I(a[1]), P(a[2]), P(a[3]), (const int*)P(a[4]), I(a[5]), (const int*)P(a[6]),
-                               (const int*)P(a[7]), P(a[8]), I(a[9]), I(a[10]), I(a[11]), I(a[12]), I(a[13]), I(a[14]),
-                               I(a[15]), I(a[16]), F(a[17]), F(a[18]), I(a[19]), I(a[20]), P(a[21]), Z(a[22]), s);
-#endif
-    default:
-      return zk_fail("zk_steplist_run: unknown entry point");
-  }
+std::vector<Op>& table() {
+  static std::vector<Op> ops = []() {
+    std::vector<Op> v;
+    v.reserve(MOST_OPS);
+    return v;
+  }();
+  return ops;
 }
+
+int enter(const char* name, int nargs, zk_packed_fn fn) {
+  if (!name || !fn || nargs < 1 || nargs > MOST_ARGS) return -1;
+  std::lock_guard<std::mutex> hold(table_lock);
+  std::vector<Op>& ops = table();
+  for (size_t i = 0; i < ops.size(); i++)
+    if (ops[i].name == name) {          // entered again (a library loaded a second time): the newer function
+      if (ops[i].nargs != nargs) return -1;
+      ops[i].fn = fn;
+      return (int)i;
+    }
+  if (ops.size() >= MOST_OPS) return -1;
+  ops.push_back(Op{name, nargs, fn});
+  return (int)ops.size() - 1;
+}
+
+// zk_gemm_bf16 tells the caller by reference into how many planes of partial sums it split K.
+// That number follows from the shape: the Python side read it when the call was written down
+// and laid the next call out accordingly; a repeated call gets a throw-away int (packed_call.h).
+#define OWN(fn) enter(#fn, zk_packed::Call<fn>::nargs, zk_packed::Call<fn>::call)
+const int entered_at_load = []() {
+  OWN(zk_embed);
+  OWN(zk_rmsnorm);
+  OWN(zk_norm_add_norm);
+  OWN(zk_gated_act);
+  OWN(zk_softcap);
+  OWN(zk_rope_cache_write);
+  OWN(zk_zero);
+  OWN(zk_gemm_plain);
+  OWN(zk_attention_plain);
+#if ZSE_ACT_BF16
+  OWN(zk_gemm_bf16);
+  OWN(zk_qkv_rope_bf16);
+  OWN(zk_attention_bf16);
+#endif
+  return 0;
+}();
+#undef OWN
 
 }  // namespace
 
 extern "C" {
 
+// Adds an entry point to the table: ``fn`` calls it from ``nargs`` argument words, the stream
+// last (the *_packed function that ZK_PACKED defines).  Returns its number, the one
+// zk_steplist_op gives for the name from now on; -1 for a bad argument.
+int zk_steplist_register(const char* name, int nargs, void* fn) { return enter(name, nargs, (zk_packed_fn)fn); }
+
 // The number of an entry point that can be written down, or -1.
 int zk_steplist_op(const char* name) {
-  for (int i = 0; i < OP_COUNT; i++) {
-#if !ZSE_ACT_BF16
-    if (i >= OP_GEMM_BF16) break;
-#endif
-    if (strcmp(OPS[i].name, name) == 0) return i;
-  }
+  if (!name) return -1;
+  std::lock_guard<std::mutex> hold(table_lock);
+  const std::vector<Op>& ops = table();
+  for (size_t i = 0; i < ops.size(); i++)
+    if (ops[i].name == name) return (int)i;
   return -1;
 }
 
@@ -160,22 +158,28 @@ int zk_steplist_size(void* list) { return list ? (int)((StepList*)list)->calls.s
 // Appends a call: ``args`` holds the entry point's arguments as 64-bit words, stream included.
 int zk_steplist_add(void* list, int op, const uint64_t* args, int nargs) {
   ZK_REQUIRE(list != nullptr && args != nullptr, "zk_steplist_add: no list");
-  ZK_REQUIRE(op >= 0 && op < OP_COUNT && nargs == OPS[op].nargs, "zk_steplist_add: wrong number of arguments");
+  {
+    std::lock_guard<std::mutex> hold(table_lock);
+    const std::vector<Op>& ops = table();
+    ZK_REQUIRE(op >= 0 && op < (int)ops.size() && nargs == ops[op].nargs, "zk_steplist_add: wrong number of arguments");
+  }
   StepCall c;
   c.op = op;
-  c.n = nargs;
   memcpy(c.a, args, sizeof(uint64_t) * nargs);
   ((StepList*)list)->calls.push_back(c);
   return 0;
 }
 
 // Launches every call of the list, in order, on ``stream``.  Stops at the first entry point
-// that refuses: its status comes back, ``*failed_at`` is its index, zk_last_error() its message.
+// that refuses: its status comes back, ``*failed_at`` is its index; its message is with the
+// library the entry point belongs to.
 int zk_steplist_run(void* list, void* stream, int* failed_at) {
   ZK_REQUIRE(list != nullptr, "zk_steplist_run: no list");
   const std::vector<StepCall>& calls = ((StepList*)list)->calls;
+  // rows are only ever added and never move: no lock while launching
+  const std::vector<Op>& ops = table();
   for (size_t i = 0; i < calls.size(); i++) {
-    const int rc = run_call(calls[i], stream);
+    const int rc = ops[calls[i].op].fn(calls[i].a, stream);
     if (rc != 0) {
       if (failed_at) *failed_at = (int)i;
       return rc;
@@ -187,7 +191,7 @@ int zk_steplist_run(void* list, void* stream, int* failed_at) {
 // The name of the entry point of call ``index`` (for error messages).
 const char* zk_steplist_name(void* list, int index) {
   if (!list || index < 0 || index >= (int)((StepList*)list)->calls.size()) return "";
-  return OPS[((StepList*)list)->calls[index].op].name;
+  return table()[((StepList*)list)->calls[index].op].name.c_str();
 }
 
 }  // extern "C"

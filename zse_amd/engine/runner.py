@@ -18,6 +18,7 @@ from __future__ import annotations
 
 import ctypes
 import inspect
+import warnings
 
 import weakref
 from dataclasses import dataclass, field
@@ -502,7 +503,12 @@ class StepRunner:
             raise
         handle = self.k.steplist_end()
         if handle is None:
-            self.use_steplists = False       # some part launches what the native side cannot repeat
+            # some part launches what the native side cannot repeat: every step of this runner is
+            # launched call by call from now on, and the reason is said, once
+            self.use_steplists = False
+            warnings.warn(f"launch lists are off for this runner: {self.k.not_written or 'an entry point'} "
+                          f"is not among the calls that can be written down (see register_kernels)",
+                          RuntimeWarning, stacklevel=2)
             return
         if len(self.steplists) >= self.MAX_STEPLISTS:
             old = next(iter(self.steplists))

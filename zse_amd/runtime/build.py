@@ -36,6 +36,18 @@ LIBRARIES: Dict[str, dict] = {
                      "device": True},
 }
 
+
+
+def register_library(name: str, sources: List[str], defines: List[str], device: bool = True) -> None:
+    """Adds a library to build: ``sources`` are files under ``zse_amd/csrc`` or absolute paths
+    (a part's own kernels live with the part), compiled with this module's flags and the
+    headers of ``zse_amd/csrc`` on the include path.  It is then built, stamped and found like
+    the three above (``ensure``, ``build``, ``build_all``)."""
+    if name in ("runtime", "kernels_f32", "kernels_bf16"):
+        raise BuildError(f"library {name} is the engine's own")
+    LIBRARIES[name] = {"sources": list(sources), "defines": list(defines), "device": bool(device)}
+
+
 DEVICE_FLAGS = [f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HOST_FLAGS = ["-O3", "-fPIC", "-std=c++17", "-Wno-unused-result"]
 
@@ -86,10 +98,10 @@ def source_digest(name: str) -> str:
     spec = LIBRARIES[name]
     h = hashlib.sha256()
     headers = [f for f in os.listdir(CSRC) if f.endswith(".h")] if os.path.isdir(CSRC) else []
-    for f in sorted(spec["sources"] + headers):
-        p = os.path.join(CSRC, f)
+    for f in sorted(spec["sources"] + headers, key=os.path.basename):
+        p = os.path.join(CSRC, f)            # an absolute path stays what it is
         if os.path.isfile(p):
-            h.update(f.encode())
+            h.update(os.path.basename(f).encode())     # not the folder: a copy of the tree elsewhere is the same source
             with open(p, "rb") as fh:
                 h.update(fh.read())
     h.update(" ".join(spec["defines"] + DEVICE_FLAGS + HOST_FLAGS).encode())
@@ -135,13 +147,13 @@ def build(name: str, verbose: bool = True, jobs: int = 0) -> str:
               file=sys.stderr, flush=True)
         threading.Thread(target=ticker, daemon=True).start()
     try:
-        objs = [os.path.join(work, os.path.splitext(s)[0] + ".o") for s in srcs]
+        objs = [os.path.join(work, os.path.splitext(os.path.basename(s))[0] + ".o") for s in srcs]
 
         def one(i):
             _run([hipcc, "-c", os.path.join(CSRC, srcs[i]), "-o", objs[i], "-I", CSRC] + flags,
                  f"compiling {srcs[i]}")
             if verbose:
-                print(f"[zse_amd]   {srcs[i]} done ({time.time() - t0:.0f} s)", file=sys.stderr,
+                print(f"[zse_amd]   {os.path.basename(srcs[i])} done ({time.time() - t0:.0f} s)", file=sys.stderr,
                       flush=True)
 
         workers = jobs or min(len(srcs), max(1, min(os.cpu_count() or 4, 16)))

@@ -173,6 +173,52 @@ BF16_KERNEL_SIGNATURES = {
 }
 
 
+@dataclass
+class KernelExtension:
+    """Kernels that a part brings along: a source file and its entry points."""
+    name: str
+    source: str                              # path of a .hip file
+    entry_points: Dict[str, list]            # entry point -> ctypes argument types, the stream last
+    written_down: bool = True
+    dtypes: Tuple[str, ...] = (F32, BF16)
+
+
+KERNEL_EXTENSIONS: Dict[str, KernelExtension] = {}
+
+
+def register_kernels(name: str, source: str, entry_points: Dict[str, list], written_down: bool = True,
+                     dtypes: Sequence[str] = (F32, BF16)) -> KernelExtension:
+    """The one call through which a part brings kernels of its own.
+
+    ``source`` is a .hip file (anywhere: beside the part).  It includes ``common.h`` and
+    ``packed_call.h`` of ``zse_amd/csrc``, says ``ZK_DEFINE_HOST_SIDE`` once, defines its entry
+    points as ``extern "C" int name(..., void* stream)`` returning 0 or a status with
+    ``zk_fail``'s message, and ``ZK_PACKED(name)`` for each.  It is compiled once per storage type
+    in ``dtypes`` (``-DZSE_ACT_BF16=0`` or ``1``, the engine's flags) into a library of its own,
+    built on first use like the engine's and found by ``__graft_entry__.build()`` too.
+    ``entry_points`` gives each entry point's ctypes argument types.  After this call every
+    ``KernelLibrary`` of a matching type has the entry points as methods (``ctx.k.name(...)``),
+    checked and raised like the engine's own.  ``written_down``: every launch reads what differs
+    between steps of one shape from device memory, so a call may be repeated from a launch list
+    (the entry points then join the native table of calls that a list can hold); False for an
+    entry point whose arguments differ from step to step: a step that calls it is launched from
+    Python every time, and the runner says so once."""
+    import os
+    if not os.path.isfile(source):
+        raise FileNotFoundError(f"kernel source {source} does not exist")
+    ext = KernelExtension(name, os.path.abspath(source), dict(entry_points), bool(written_down),
+                          tuple(canonical_dtype(d) for d in dtypes))
+    KERNEL_EXTENSIONS[name] = ext
+    for d in ext.dtypes:
+        build.register_library(_extension_library(name, d), [ext.source],
+                               ["-DZSE_ACT_BF16=1" if d == BF16 else "-DZSE_ACT_BF16=0"], device=True)
+    return ext
+
+
+def _extension_library(name: str, dtype: str) -> str:
+    return f"ext_{name}_{'bf16' if dtype == BF16 else 'f32'}"
+
+
 class KernelLibrary:
     """One built kernel library; calling ``lib.zk_x(...)`` raises on a non-zero status."""
 
@@ -222,12 +268,51 @@ class KernelLibrary:
         want = 1 if dtype == BF16 else 0
         if self._dll.zk_act_is_bf16() != want:
             raise DeviceError(f"{path} was built for the other storage type")
+        self._attached: Dict[str, object] = {}      # extension name -> its loaded library
+        self.attach_extensions()
 
     def has(self, name: str) -> bool:
         return hasattr(self, name)
 
-    def _wrap(self, name, fn):
-        dll = self._dll
+    def attach_extensions(self) -> None:
+        """Loads the libraries of every registered extension that this library has not met yet
+        (built first if need be), makes their entry points methods of this object and enters
+        those that may be written down into the native table of a launch list's calls."""
+        for ext in list(KERNEL_EXTENSIONS.values()):
+            if self.dtype not in ext.dtypes or self._attached.get(ext.name) is ext:
+                continue
+            path = build.ensure(_extension_library(ext.name, self.dtype))
+            dll = C.CDLL(path)
+            dll.zk_last_error.restype = C.c_char_p
+            if dll.zk_act_is_bf16() != (1 if self.dtype == BF16 else 0):
+                raise DeviceError(f"{path} was built for the other storage type")
+            for name, args in ext.entry_points.items():
+                try:
+                    fn = getattr(dll, name)
+                except AttributeError:
+                    raise DeviceError(f"{path} (built from {ext.source}) lacks {name}") from None
+                fn.argtypes, fn.restype = list(args), C.c_int
+                setattr(self, name, self._wrap(name, fn, dll))
+                self._op_ids.pop(name, None)
+                if ext.written_down:
+                    try:
+                        packed, nargs = getattr(dll, name + "_packed"), getattr(dll, name + "_nargs")
+                    except AttributeError:
+                        raise DeviceError(f"{ext.source}: ZK_PACKED({name}) is missing, which an entry point "
+                                          f"that may be written down needs") from None
+                    nargs.restype = C.c_int
+                    if nargs() != len(args):
+                        raise DeviceError(f"{name}: {len(args)} argument types were registered, the entry point "
+                                          f"takes {nargs()}")
+                    op = self._dll.zk_steplist_register(name.encode(), len(args), C.cast(packed, C.c_void_p))
+                    if op < 0:
+                        raise DeviceError(f"{name} could not be entered into the table of written-down calls")
+                self._owner_of[name] = dll
+            self._attached[ext.name] = ext
+            self._keep_alive.append(dll)
+
+    def _wrap(self, name, fn, dll=None):
+        dll = dll or self._dll
         lib = self
 
         def call(*a):
@@ -251,6 +336,11 @@ class KernelLibrary:
         d.zk_steplist_run.restype = C.c_int
         d.zk_steplist_run.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_int)]
         d.zk_steplist_name.restype, d.zk_steplist_name.argtypes = C.c_char_p, [C.c_void_p, C.c_int]
+        d.zk_steplist_register.restype = C.c_int
+        d.zk_steplist_register.argtypes = [C.c_char_p, C.c_int, C.c_void_p]
+        self._owner_of: Dict[str, object] = {}      # entry point of an extension -> its library
+        self._keep_alive = []
+        self.not_written: Optional[str] = None      # the entry point that kept the last list from being written
         self._writing = None          # the list being written, while a step runs call by call
         self._writable = True
         self._op_ids: Dict[str, int] = {}
@@ -277,8 +367,9 @@ class KernelLibrary:
         rc = self._dll.zk_steplist_run(handle, stream, C.byref(at))
         if rc != 0:
             name = self._dll.zk_steplist_name(handle, at.value).decode()
+            owner = self._owner_of.get(name, self._dll)
             raise DeviceError(f"{name} (call {at.value} of a written-down step) failed ({rc}): "
-                              f"{self._dll.zk_last_error().decode()}")
+                              f"{owner.zk_last_error().decode()}")
 
     def steplist_destroy(self, handle: int) -> None:
         self._dll.zk_steplist_destroy(handle)
@@ -291,6 +382,8 @@ class KernelLibrary:
         if op is None:
             op = self._op_ids[name] = self._dll.zk_steplist_op(name.encode())
         if op < 0 or not self._writable:
+            if op < 0 and self._writable:
+                self.not_written = name
             self._writable = False          # an entry point the native side cannot call again
             return
         words = (C.c_uint64 * len(args))()
@@ -384,6 +477,10 @@ class Runtime:
         if dtype not in self._kernels:
             name = "kernels_bf16" if dtype == BF16 else "kernels_f32"
             self._kernels[dtype] = KernelLibrary(build.ensure(name), dtype)
+        elif len(self._kernels[dtype]._attached) != len(KERNEL_EXTENSIONS) or \
+                any(self._kernels[dtype]._attached.get(n) is not e for n, e in KERNEL_EXTENSIONS.items()
+                    if dtype in e.dtypes):
+            self._kernels[dtype].attach_extensions()      # kernels registered since the library was loaded
         return self._kernels[dtype]
 
     # -- memory
