@@ -103,15 +103,14 @@ def test_norm_ffn_embedding_head_alone(rt, tiny_folders, name, dtype):
     assert np.abs(rt.download(out) - want).max() < tol * max(1.0, np.abs(want).max())
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
-def test_attention_mixer_alone(rt, tiny_folders, name, dtype):
+def mixer_alone(rt, tiny_folders, name, dtype, build, before_rotation=None):
     """The mixer of a sliding layer and of a global one over a cache of their own: a portion of a
-    prompt, then single tokens, against the plain rope + attention + projections."""
+    prompt, then single tokens, against the plain rope + attention + projections.
+    ``build(spec)`` makes the mixer; ``before_rotation(q, k)`` is what the plain side does to
+    queries and keys [T, heads, hd] between the products and the rotation."""
     from zse_amd.engine.model import CallCache
     from zse_amd.engine.runner import GroupView
     from zse_amd.models.gemma2 import Gemma2Config, gemma2_plan
-    from zse_amd.parts import build_part
     cfg = TINY[name][0]
     c = P.read_config(cfg)
     plan = gemma2_plan(Gemma2Config.from_dict(cfg))
@@ -122,7 +121,7 @@ def test_attention_mixer_alone(rt, tiny_folders, name, dtype):
     T, H, bs, pages = 45, cfg["hidden_size"], 8, 12
     for layer in (0, 1):
         spec = plan.layers[layer].mixer
-        mixer = build_part("mixer", spec)
+        mixer = build(spec)
         for p in [mixer] + mixer.children():
             p.load(src, rt, dtype)
         x = rounded(rng.normal(size=(T, H)), dtype)
@@ -131,6 +130,8 @@ def test_attention_mixer_alone(rt, tiny_folders, name, dtype):
         q = (x @ w[spec.names["q"]].T.astype(f64)).reshape(T, c["nh"], c["hd"])
         kk = (x @ w[spec.names["k"]].T.astype(f64)).reshape(T, c["nkv"], c["hd"])
         vv = (x @ w[spec.names["v"]].T.astype(f64)).reshape(T, c["nkv"], c["hd"])
+        if before_rotation is not None:
+            q, kk = before_rotation(q, kk)
         o = P.attention(P.rope(q, pos, c["theta"], f64), P.rope(kk, pos, c["theta"], f64), vv, pos,
                         c["qpas"] ** -0.5, c["attn_cap"], spec.window, f64)
         want = o.reshape(T, -1) @ w[spec.names["o"]].T.astype(f64)
@@ -156,6 +157,33 @@ def test_attention_mixer_alone(rt, tiny_folders, name, dtype):
             got.append(rt.download_f32(mixer.forward(ctx, up(rt, x[start:start + n], dtype), cache)))
         got = np.concatenate(got)
         assert np.abs(got - want).max() < tol * max(1.0, np.abs(want).max()), f"layer {layer}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_attention_mixer_alone(rt, tiny_folders, name, dtype):
+    from zse_amd.parts import build_part
+    mixer_alone(rt, tiny_folders, name, dtype, lambda spec: build_part("mixer", spec))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_mixer_that_differs_between_product_and_rotation(rt, tiny_folders, dtype):
+    """Attention whose queries and keys are scaled to unit length, head by head, before they are
+    rotated: a subclass of the framework's attention that overrides one method and brings one
+    kernel; product, rotation, cache, attention kernels and output product stay the framework's."""
+    import toy_kernels  # noqa: F401  (registers zk_toy_head_norm)
+    from zse_amd.parts.attention import PagedAttention
+
+    class UnitLengthAttention(PagedAttention):
+        def between_product_and_rotation(self, ctx, qkv):
+            s = self.spec
+            ctx.rt.kernels(ctx.dtype).zk_toy_head_norm(qkv.ptr, qkv.shape[0], qkv.shape[1],
+                                                       s.num_heads + s.num_kv_heads, s.head_dim, ctx.stream)
+
+    def unit(q, k):
+        return (q / np.linalg.norm(q, axis=-1, keepdims=True), k / np.linalg.norm(k, axis=-1, keepdims=True))
+
+    mixer_alone(rt, tiny_folders, "B", dtype, UnitLengthAttention, before_rotation=unit)
 
 
 def test_toy_mixer_with_state_is_registered_built_and_stepped(rt):

@@ -138,6 +138,25 @@ def test_names_match_with_or_without_model_prefix(tmp_path):
     assert len(check_folder(d, reqs_of(TINY_A))) == len(w)
 
 
+def test_the_optional_prefix_is_the_plans_to_name(tmp_path):
+    """Which prefix a checkpoint may leave out is data of the plan (``optional_prefixes``), not a
+    word in the loader: with another architecture's prefix the same file is matched, with none
+    the names must be exact."""
+    from zse_amd.parts.base import TensorReq
+    from zse_amd.weights.loader import WeightError, check_entries
+    d = str(tmp_path / "m")
+    os.makedirs(d)
+    st.write_file(os.path.join(d, "model.safetensors"),
+                  {"transformer.wte": ("F32", np.zeros((4, 2), np.float32)), "h.0.w": ("F32", np.zeros((2, 2), np.float32))})
+    reqs = [TensorReq("wte", (4, 2)), TensorReq("transformer.h.0.w", (2, 2))]
+    entries = st.index_folder(d)
+    got = check_entries(entries, reqs, prefixes=("transformer.",))
+    assert sorted(got) == ["h.0.w", "wte"]
+    with pytest.raises(WeightError) as e:
+        check_entries(entries, reqs, prefixes=())
+    assert sorted(e.value.missing) == ["transformer.h.0.w", "wte"] and sorted(e.value.unexpected) == ["h.0.w", "transformer.wte"]
+
+
 def test_untied_model_wants_lm_head(tmp_path):
     cfg = dict(TINY_A, tie_word_embeddings=False)
     d = write_random_model(str(tmp_path / "m"), cfg, seed=0, dtype="float32")

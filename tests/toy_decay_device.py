@@ -2,18 +2,12 @@
 beside this file), brought to the framework through ``register_kernels``: the framework
 compiles it, makes it a method of the kernel library and lets launch lists and captured
 graphs repeat it.  Nothing under ``zse_amd/`` knows of it."""
-import ctypes as C
-import os
-
-from zse_amd.parts import Part, StateNeed, TensorReq, register_kernels, register_part
-from zse_amd.parts.ops import linear
-
 from dataclasses import dataclass
 
-_VP, _I, _F = C.c_void_p, C.c_int, C.c_float
+from zse_amd.parts import Part, StateNeed, TensorReq, register_part
+from zse_amd.parts.ops import linear
 
-register_kernels("toy_decay", os.path.join(os.path.dirname(os.path.abspath(__file__)), "toy_decay.hip"),
-                 {"zk_toy_decay": [_VP, _VP, _VP, _I, _I, _VP, _VP, _I, _I, _F, _VP]})
+import toy_kernels  # noqa: F401  (registers zk_toy_decay)
 
 
 @dataclass(frozen=True)

@@ -125,6 +125,9 @@ class ModelPlan:
     final_norm: Any
     head: HeadSpec
     ignored_tensors: Tuple[str, ...] = ()   # checkpoint names that may be present and are not used
+    # what a checkpoint may or may not put in front of a tensor's name: "model.layers.0..." and
+    # "layers.0..." are the same tensor (format/arch/gemma2.py:50-55 accepts both)
+    optional_prefixes: Tuple[str, ...] = ("model.",)
 
     def describe(self) -> List[str]:
         out = []

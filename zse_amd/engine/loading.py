@@ -19,7 +19,8 @@ def load_model(model_dir: str, dtype: str, rt: Optional[Runtime] = None, tuned: 
     arch, config = load_config(model_dir)
     model = Model(arch.plan(config))
     model.config = config
-    src = CheckpointWeights(rt, dtype, model_dir, model.tensor_reqs(), model.plan.ignored_tensors, tuned=tuned)
+    src = CheckpointWeights(rt, dtype, model_dir, model.tensor_reqs(), model.plan.ignored_tensors, tuned=tuned,
+                            prefixes=model.plan.optional_prefixes)
     model.load(src, rt, dtype)
     model.tuned = bool(tuned)
     rt.sync()
@@ -38,7 +39,8 @@ def random_model(config: dict, dtype: str, seed: int = 0, std: float = 0.02, gai
     typed = arch.config_from_dict(config)
     model = Model(arch.plan(typed))
     model.config = typed
-    src = RandomWeights(rt, dtype, model.tensor_reqs(), seed, std, gain_std, tuned=tuned, std_of=std_of)
+    src = RandomWeights(rt, dtype, model.tensor_reqs(), seed, std, gain_std, tuned=tuned, std_of=std_of,
+                        prefixes=model.plan.optional_prefixes)
     model.load(src, rt, dtype)
     model.tuned = bool(tuned)
     rt.sync()

@@ -93,6 +93,14 @@ class PagedAttention(Part):
             need = (need + 255) // 256 * 256 + min(extra, self.PORTION_RANGES_BYTES)
         return need
 
+    def between_product_and_rotation(self, ctx, qkv: Tensor) -> None:
+        """A mixer that differs from this one only in what it does to queries and keys before
+        they are rotated and stored (a norm over each head, say) overrides this and changes
+        ``qkv`` in place: rows are tokens, a row holds the query heads, then the key heads, then
+        the value heads (the last two absent in a mixer that reads another entry's cache), each
+        ``head_dim`` wide.  Everything else of the mixer stays as it is; the product that
+        rotates and stores its own results is then not used, since this step lies in between."""
+
     def forward(self, ctx, x: Tensor, cache) -> Tensor:
         s, k = self.spec, ctx.k
         T = x.shape[0]
@@ -101,7 +109,8 @@ class PagedAttention(Part):
         width = (nh + 2 * n_store) * hd
         g = ctx.group(cache.group)
         tables = self.position.rotary_tables()
-        if (tables is not None and tuned_gemm(ctx, s.hidden_size) and k.has("zk_qkv_rope_bf16")
+        hooked = type(self).between_product_and_rotation is not PagedAttention.between_product_and_rotation
+        if (not hooked and tables is not None and tuned_gemm(ctx, s.hidden_size) and k.has("zk_qkv_rope_bf16")
                 and k.zk_qkv_rope_bf16_supports(T, s.hidden_size, hd, tables[1])):
             # few decoded tokens: the product rotates and stores its own results
             qkv = ctx.alloc((T, width))
@@ -112,6 +121,8 @@ class PagedAttention(Part):
                                ctx.stream)
         else:
             qkv = linear(ctx, x, self.w_qkv, ctx.alloc((T, width)))
+            if hooked:
+                self.between_product_and_rotation(ctx, qkv)
             if tables is None:
                 self.position.apply(ctx, qkv, nh, n_store, hd)
                 inv_freq, rotary_dim = 0, 0

@@ -48,15 +48,23 @@ class WeightError(ValueError):
         super().__init__("checkpoint does not match the model: " + "; ".join(lines))
 
 
-def _strip(name: str) -> str:
-    return name[6:] if name.startswith("model.") else name
+DEFAULT_PREFIXES = ("model.",)
 
 
-def merge_reqs(reqs: Iterable[TensorReq]) -> Dict[str, TensorReq]:
+def _strip(name: str, prefixes: Sequence[str] = DEFAULT_PREFIXES) -> str:
+    """The name without the first of ``prefixes`` it begins with: checkpoints of one
+    architecture come with and without such a prefix (``ModelPlan.optional_prefixes``)."""
+    for p in prefixes:
+        if p and name.startswith(p):
+            return name[len(p):]
+    return name
+
+
+def merge_reqs(reqs: Iterable[TensorReq], prefixes: Sequence[str] = DEFAULT_PREFIXES) -> Dict[str, TensorReq]:
     """One entry per name; a name asked for twice (tied weights) must agree in shape."""
     out: Dict[str, TensorReq] = {}
     for r in reqs:
-        key = _strip(r.name)
+        key = _strip(r.name, prefixes)
         if key in out and out[key].shape != tuple(r.shape):
             raise ValueError(f"tensor {r.name} is asked for with shapes {out[key].shape} and {r.shape}")
         out.setdefault(key, TensorReq(r.name, tuple(r.shape), r.role, r.init_std))
@@ -64,14 +72,14 @@ def merge_reqs(reqs: Iterable[TensorReq]) -> Dict[str, TensorReq]:
 
 
 def check_entries(entries: Dict[str, st.TensorEntry], reqs: Iterable[TensorReq],
-                  ignored: Sequence[str] = ()) -> Dict[str, st.TensorEntry]:
+                  ignored: Sequence[str] = (), prefixes: Sequence[str] = DEFAULT_PREFIXES) -> Dict[str, st.TensorEntry]:
     """Match checkpoint entries to requests; raises ``WeightError`` with every finding.
     Returns stripped name -> entry."""
-    want = merge_reqs(reqs)
+    want = merge_reqs(reqs, prefixes)
     have = {}
     for name, e in entries.items():
-        have[_strip(name)] = e
-    skip = {_strip(n) for n in ignored}
+        have[_strip(name, prefixes)] = e
+    skip = {_strip(n, prefixes) for n in ignored}
     missing = [want[k].name for k in want if k not in have]
     unexpected = [have[k].name for k in have if k not in want and k not in skip]
     wrong_shape = [(have[k].name, have[k].shape, want[k].shape) for k in want
@@ -83,15 +91,17 @@ def check_entries(entries: Dict[str, st.TensorEntry], reqs: Iterable[TensorReq],
     return {k: have[k] for k in want}
 
 
-def check_folder(model_dir: str, reqs: Iterable[TensorReq], ignored: Sequence[str] = ()):
-    return check_entries(st.index_folder(model_dir), reqs, ignored)
+def check_folder(model_dir: str, reqs: Iterable[TensorReq], ignored: Sequence[str] = (),
+                 prefixes: Sequence[str] = DEFAULT_PREFIXES):
+    return check_entries(st.index_folder(model_dir), reqs, ignored, prefixes)
 
 
 class _Source:
     """Common part of weight sources: caching, so that tied names share one tensor."""
 
-    def __init__(self, rt, dtype: str, tuned: bool = True):
+    def __init__(self, rt, dtype: str, tuned: bool = True, prefixes: Sequence[str] = DEFAULT_PREFIXES):
         self.rt = rt
+        self.prefixes = tuple(prefixes)
         self.dtype = dtype
         self.tuned = bool(tuned)      # parts may ask for layouts that only the tuned kernels read
         self.k = rt.kernels(dtype)
@@ -108,10 +118,10 @@ class _Source:
     def matrix(self, names: Sequence[str], strip: bool = False) -> Tensor:
         """The named 2-D tensors stacked along rows, in the compute type.  ``strip``: in strip
         layout (rows padded to a multiple of 16; the shape stays the logical one)."""
-        key = ("s" if strip else "m",) + tuple(_strip(n) for n in names)
+        key = ("s" if strip else "m",) + tuple(_strip(n, self.prefixes) for n in names)
         if key not in self._cache and strip:
             rows = self.matrix(names)
-            self._cache.pop(("m",) + tuple(_strip(n) for n in names))
+            self._cache.pop(("m",) + tuple(_strip(n, self.prefixes) for n in names))
             self.bytes_on_device -= rows.nbytes
             n, k = rows.shape
             out = self.rt.empty(((n + 15) // 16 * 16, k), self.dtype)
@@ -134,7 +144,7 @@ class _Source:
         return self._cache[key]
 
     def vector(self, name: str) -> Tensor:
-        key = ("v", _strip(name))
+        key = ("v", _strip(name, self.prefixes))
         if key not in self._cache:
             out = self.rt.empty(self._shape(name), F32)
             self._fill(name, out, 0)
@@ -147,16 +157,16 @@ class CheckpointWeights(_Source):
     """Tensors of a checked model folder, copied and converted on the device."""
 
     def __init__(self, rt, dtype: str, model_dir: str, reqs: Iterable[TensorReq],
-                 ignored: Sequence[str] = (), tuned: bool = True):
-        super().__init__(rt, dtype, tuned)
-        self.entries = check_folder(model_dir, reqs, ignored)
+                 ignored: Sequence[str] = (), tuned: bool = True, prefixes: Sequence[str] = DEFAULT_PREFIXES):
+        super().__init__(rt, dtype, tuned, prefixes)
+        self.entries = check_folder(model_dir, reqs, ignored, prefixes)
         self._staging = None
 
     def _shape(self, name):
-        return self.entries[_strip(name)].shape
+        return self.entries[_strip(name, self.prefixes)].shape
 
     def _fill(self, name: str, dst: Tensor, dst_kind: int):
-        e = self.entries[_strip(name)]
+        e = self.entries[_strip(name, self.prefixes)]
         arr = st.map_tensor(e)
         same = (e.dtype == "F32" and dst.dtype == F32) or (e.dtype == "BF16" and dst.dtype == BF16)
         if same:
@@ -187,30 +197,31 @@ class RandomWeights(_Source):
     N(0, gain_std); each value is a function of (seed, tensor name, index)."""
 
     def __init__(self, rt, dtype: str, reqs: Iterable[TensorReq], seed: int, std: float = 0.02,
-                 gain_std: float = 0.1, tuned: bool = True, std_of=None):
-        super().__init__(rt, dtype, tuned)
-        self.reqs = merge_reqs(reqs)
+                 gain_std: float = 0.1, tuned: bool = True, std_of=None,
+                 prefixes: Sequence[str] = DEFAULT_PREFIXES):
+        super().__init__(rt, dtype, tuned, prefixes)
+        self.reqs = merge_reqs(reqs, prefixes)
         self.seed, self.std, self.gain_std = int(seed), float(std), float(gain_std)
         self.std_of = dict(std_of or {})
 
     def _shape(self, name):
-        return self.reqs[_strip(name)].shape
+        return self.reqs[_strip(name, self.prefixes)].shape
 
     def _fill(self, name: str, dst: Tensor, dst_kind: int):
         from .normal import stream_of
         from .random_init import deviation_of
-        r = self.reqs[_strip(name)]
+        r = self.reqs[_strip(name, self.prefixes)]
         std = deviation_of(r, self.std, self.gain_std, self.std_of)
         if dst_kind == 0 and self.dtype == BF16:
             # a vector kept as float32 in a bfloat16 model holds what a bfloat16 checkpoint
             # would: values rounded to bfloat16 (so the model equals the folder written on the host)
             tmp = self.rt.empty((dst.numel,), BF16)
-            self.k.zk_fill_normal(tmp.ptr, 1, dst.numel, self.seed, stream_of(_strip(name)), 0.0, std,
+            self.k.zk_fill_normal(tmp.ptr, 1, dst.numel, self.seed, stream_of(_strip(name, self.prefixes)), 0.0, std,
                                   self.rt.stream)
             self.k.zk_convert(tmp.ptr, SRC_TAGS["BF16"], dst.ptr, 0, dst.numel, self.rt.stream)
             self.rt.sync()
             return
-        self.k.zk_fill_normal(dst.ptr, dst_kind, dst.numel, self.seed, stream_of(_strip(name)), 0.0, std,
+        self.k.zk_fill_normal(dst.ptr, dst_kind, dst.numel, self.seed, stream_of(_strip(name, self.prefixes)), 0.0, std,
                               self.rt.stream)
 
     def close(self):

@@ -34,10 +34,11 @@ def deviation_of(req, std: float, gain_std: float, std_of=None) -> float:
     return float(s)
 
 
-def random_tensors(reqs, seed: int, std: float, gain_std: float, std_of=None):
+def random_tensors(reqs, seed: int, std: float, gain_std: float, std_of=None, prefixes=None):
     """{name: float32 array} for every tensor the parts ask for (one draw per name)."""
+    merged = merge_reqs(reqs) if prefixes is None else merge_reqs(reqs, prefixes)
     return {r.name: normal_tensor(r.shape, seed, key, 0.0, deviation_of(r, std, gain_std, std_of))
-            for key, r in merge_reqs(reqs).items()}
+            for key, r in merged.items()}
 
 
 def write_random_model(out_dir: str, config: dict, seed: int = 0, std: float = 0.02,
@@ -53,7 +54,7 @@ def write_random_model(out_dir: str, config: dict, seed: int = 0, std: float = 0
     arch = resolve_architecture(config)
     typed = arch.config_from_dict(config)
     model = Model(arch.plan(typed))
-    tensors = random_tensors(model.tensor_reqs(), seed, std, gain_std, std_of)
+    tensors = random_tensors(model.tensor_reqs(), seed, std, gain_std, std_of, model.plan.optional_prefixes)
     if dtype in ("bfloat16", "bf16"):
         packed = {n: ("BF16", st.f32_to_bf16_bits(a)) for n, a in tensors.items()}
     elif dtype in ("float32", "fp32"):
