@@ -19,9 +19,14 @@ same weights made on the host, and at every batch size that is timed the full mo
 steps through the timed path (captured graphs or launch lists, ids fed on the device) must pick
 the same tokens as steps launched call by call.  A failed check ends the run with an error.
 
-``--workload`` runs one of the two larger workloads through ``Engine.generate`` instead, end to
-end: 9b = 32 requests with prompts of 128 to 4,096 tokens, 256 greedy tokens each, portions of
-512; 27b = 8 prompts of 8,192 tokens, 128 tokens each at temperature 1.0, seed 3.
+The same run then goes on to further sizes (``--quick`` leaves them out): the 2B shapes decoding
+at a context of 8,192, and the 9B and 27B shapes (decode at batch 8, a 2,048-token prefill, and
+their serving workloads through ``Engine.generate``, end to end: 9b = 32 requests with prompts of
+128 to 4,096 tokens, 256 greedy tokens each, portions of 512; 27b = 8 prompts of 8,192 tokens,
+128 tokens each at temperature 1.0, seed 3).  They land in ``points`` (tokens a second) and, with
+their times and fractions of the peaks, in ``further``.  ``--workload 9b|27b`` runs one workload
+alone.  What a step has to read and to compute is read off the model's parts (``Model.flops``,
+``Model.cache_bytes_read``, the bytes of its weights), not written down here per architecture.
 """
 import argparse
 import json
@@ -49,38 +54,6 @@ GEMMA2_9B = dict(GEMMA2_2B, num_hidden_layers=42, hidden_size=3584, num_attentio
 GEMMA2_27B = dict(GEMMA2_2B, num_hidden_layers=46, hidden_size=4608, num_attention_heads=32, num_key_value_heads=16,
                   head_dim=128, query_pre_attn_scalar=144, intermediate_size=36864)
 MODELS = {"2b": GEMMA2_2B, "9b": GEMMA2_9B, "27b": GEMMA2_27B}
-
-
-def weight_bytes(cfg, item=2):
-    H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
-    nh, nkv, hd, L = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["num_hidden_layers"]
-    per_layer = (nh + 2 * nkv) * hd * H + H * nh * hd + 3 * I * H
-    return (L * per_layer + V * H) * item
-
-
-def cache_bytes(cfg, ctx, item=2):
-    """Bytes of keys and values one request's decode step reads at context ``ctx``."""
-    nkv, hd, L, W = cfg["num_key_value_heads"], cfg["head_dim"], cfg["num_hidden_layers"], cfg["sliding_window"]
-    total = 0
-    for l in range(L):
-        seen = min(ctx, W) if (l % 2 == 0 and W) else ctx
-        total += 2 * nkv * hd * seen * item
-    return total
-
-
-def prefill_flops(cfg, T, start=0):
-    """Flops of a step that brings tokens [start, start + T) of one request and wants one row."""
-    H, I, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
-    nh, nkv, hd, L, W = (cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"],
-                         cfg["num_hidden_layers"], cfg["sliding_window"])
-    per_layer = (nh + 2 * nkv) * hd * H + H * nh * hd + 3 * I * H
-    gemm = 2.0 * T * per_layer * L
-    attn = 0.0
-    for l in range(L):
-        w = W if (l % 2 == 0 and W) else start + T
-        keys = sum(min(i + 1, w) for i in range(start, start + T))
-        attn += 4.0 * nh * hd * keys
-    return gemm + attn + 2.0 * V * H
 
 
 def log(msg):
@@ -220,7 +193,8 @@ def check_decode_path(model, rt, vocab, B, use_graphs):
 
 
 # ------------------------------------------------------------------ workloads through the engine
-def run_workload(name, a):
+def run_workload(name, a, model=None):
+    """One of the two larger workloads through ``Engine.generate``; returns its record."""
     from zse_amd.engine.engine import Engine
     from zse_amd.engine.loading import random_model
     from zse_amd.runtime.device import Runtime
@@ -234,8 +208,9 @@ def run_workload(name, a):
         cfg["max_position_embeddings"] = 8192 + 128
     rt = Runtime.get()
     t0 = time.time()
-    model = random_model(cfg, "bfloat16", seed=0, std=0.02, gain_std=0.1, rt=rt)
-    log(f"{name}: model ready in {time.time() - t0:.1f} s, {model.weight_bytes / 1e9:.2f} GB of weights")
+    if model is None:
+        model = random_model(cfg, "bfloat16", seed=0, std=0.02, gain_std=0.1, rt=rt)
+        log(f"{name}: model ready in {time.time() - t0:.1f} s, {model.weight_bytes / 1e9:.2f} GB of weights")
     rng = np.random.default_rng(0)
     V, page = cfg["vocab_size"], 16
     if name == "9b":
@@ -299,7 +274,144 @@ def run_workload(name, a):
         "tpot_ms_mean": round(float(np.mean(st.tpot_ms)), 3),
     }
     eng.close()
-    print(json.dumps(res), flush=True)
+    return res
+
+
+class Timed:
+    """A model on a runner sized for the batches and the context that are timed."""
+
+    def __init__(self, model, rt, cfg, max_b, context, prefill_tokens, graphs):
+        from zse_amd.engine.runner import StepRunner
+        from zse_amd.sampling.sampler import DeviceSampler
+        self.model, self.rt, self.cfg, self.context, self.T = model, rt, cfg, context, prefill_tokens
+        self.V, page = cfg["vocab_size"], 16
+        longest = max(context, prefill_tokens)       # a prompt longer than the decode context still fits
+        self.runner = StepRunner(model, rt, "bfloat16", page_size=page,
+                                 num_pages=max(max_b * (-(-context // page) + 1), -(-longest // page)) + 8,
+                                 max_seqs=max_b, max_batch_tokens=max(prefill_tokens, max_b), max_model_len=longest,
+                                 use_graphs=graphs)
+        self.sampler = DeviceSampler(rt, self.runner.k, max_b)
+        self.rng = np.random.default_rng(0)
+        # Steady state is what is measured.  For about a second after a process has allocated tens
+        # of GB (the cache slabs, just now) kernels that wait for memory rather than stream from it
+        # run up to 17 % slower (the o and down products of a decode step: 10.1 instead of 8.7 us;
+        # steps at batch 1 and 8 by 3 to 4 %); later steps of the same process do not, whatever was
+        # done meanwhile.  So the timed work starts two seconds after the allocations.
+        rt.sync()
+        time.sleep(2.0)
+
+    def close(self):
+        self.runner.close()
+        self.runner = self.sampler = None
+
+    def prefill(self, portion=None, repeats=3):
+        """One prompt of ``self.T`` tokens, whole or in portions of ``portion`` tokens, logits of
+        its last token wanted: (seconds, flops), the median of ``repeats`` after one untimed."""
+        from zse_amd.engine.runner import StepEntry
+        T, runner, rt = self.T, self.runner, self.rt
+        portion = portion or T
+        times = []
+        for i in range(repeats + 1):
+            toks = self.rng.integers(0, self.V, T).tolist()
+            rt.sync()
+            t1 = time.perf_counter()
+            for at in range(0, T, portion):
+                n = min(portion, T - at)
+                runner.step([StepEntry("p", toks[at:at + n], [n - 1] if at + n == T else [])], download=False)
+            rt.sync()
+            times.append(time.perf_counter() - t1)
+            runner.finish("p")
+        flops = sum(self.model.flops([(at, min(portion, T - at))], 1 if at + portion >= T else 0)
+                    for at in range(0, T, portion))
+        return float(np.median(times[1:])), flops
+
+    def decode(self, B, steps, warmup):
+        """``steps`` decode steps of ``B`` requests that end at the full context: (tokens a
+        second, seconds a step, bytes a step has to read, how the steps were launched)."""
+        from zse_amd.engine.runner import StepEntry
+        from zse_amd.sampling.sampler import SamplingParams
+        runner, rt, sampler, rng, V = self.runner, self.rt, self.sampler, self.rng, self.V
+        ctx0 = self.context - steps - warmup
+        reqs = [f"d{B}_{i}" for i in range(B)]
+        for r in reqs:                       # fill the cache through real prefill steps
+            left = ctx0
+            while left > 0:
+                n = min(left, self.T)
+                runner.step([StepEntry(r, rng.integers(0, V, n).tolist(), [])], download=False)
+                left -= n
+        first = rng.integers(0, V, B).tolist()
+        rows = [{"params": SamplingParams(temperature=0.0), "u": 0.0} for _ in range(B)]
+        # As the engine decodes: the sampling kernel leaves the ids on the device, the next step
+        # takes them from there, and the host reads them four steps at a time (it has to, for
+        # stop tokens) while the next steps are already enqueued.
+        sampler.prepare_run(rows, [[0.0] * B])
+        pending, fed = [], None
+
+        def one():
+            nonlocal fed
+            toks = first if fed is None else [0] * B
+            logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(reqs, toks)], download=False,
+                                 tokens_from=fed)
+            ids = sampler.sample_deferred(logits, 0)
+            fed = ids.device_ptr
+            pending.append(ids)
+            if len(pending) == 4:
+                for p in pending:
+                    p.result()
+                pending.clear()
+        lists0 = runner.steplist_runs
+        for _ in range(warmup):
+            one()
+        rt.sync()
+        t1 = time.perf_counter()
+        for _ in range(steps):
+            one()
+        rt.sync()
+        dt = time.perf_counter() - t1
+        for r in reqs:
+            runner.finish(r)
+        how = "graph" if runner._graph_bucket([StepEntry(r, [0], [0]) for r in reqs]) else \
+            ("launch list" if runner.steplist_runs > lists0 else "call by call")
+        mean_ctx = int(self.context - steps / 2.0)
+        byts = self.model.weight_bytes + B * self.model.cache_bytes_read(mean_ctx, 2)
+        return B * steps / dt, dt / steps, byts, how
+
+
+def shape_of(cfg, full_layers):
+    return {"layers": cfg["num_hidden_layers"], "layers_full": full_layers, "hidden": cfg["hidden_size"],
+            "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+            "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"], "sliding_window": cfg["sliding_window"]}
+
+
+def further_model(name, a, rt, peak_bw, peak_fl):
+    """Decode at batch 8, a 2,048-token prefill and the serving workload of one of the larger
+    models, each with its fraction of the nominal peak."""
+    from zse_amd.engine.loading import random_model
+    cfg = dict(MODELS[name], max_position_embeddings=8192 + 128)
+    t0 = time.time()
+    model = random_model(cfg, "bfloat16", seed=0, std=0.02, gain_std=0.1, rt=rt)
+    log(f"{name}: model ready in {time.time() - t0:.1f} s, {model.weight_bytes / 1e9:.2f} GB of weights")
+    same = check_decode_path(model, rt, cfg["vocab_size"], 8, not a.no_graphs)
+    if not same:
+        raise SystemExit(f"bench.py: {name}: the timed decode path does not pick the tokens of eager steps")
+    t = Timed(model, rt, cfg, 8, a.context, a.prefill_tokens, not a.no_graphs)
+    pre_s, pf = t.prefill()
+    tok_s, step_s, byts, how = t.decode(8, max(16, a.steps // 2), max(4, a.warmup // 2))
+    t.close()
+    out = {"config": dict(shape_of(cfg, cfg["num_hidden_layers"]), weights_gb=round(model.weight_bytes / 1e9, 2)),
+           "decode_b8": {"value": round(tok_s, 1), "ms_per_step": round(step_s * 1e3, 3), "context": a.context,
+                         "launched": how, "roofline_frac": round(byts / step_s / PEAK_HBM, 4),
+                         "gbs": round(byts / step_s / 1e9, 1)},
+           "prefill": {"value": round(a.prefill_tokens / pre_s, 1), "tokens": a.prefill_tokens, "ms": round(pre_s * 1e3, 3),
+                       "frac": round(pf / pre_s / PEAK_FLOPS["bf16"], 4)}}
+    log(f"{name}: decode batch 8 {step_s * 1e3:.3f} ms/step ({out['decode_b8']['roofline_frac']} of 8 TB/s), "
+        f"prefill {pre_s * 1e3:.2f} ms ({out['prefill']['frac']} of 2.5 PFLOP/s)")
+    w = run_workload(name, a, model=model)
+    out["workload"] = {k: w[k] for k in ("value", "unit", "workload", "seconds", "generated_tokens", "prompt_tokens",
+                                         "all_tokens_per_s", "steps", "preemptions", "by_kind", "ttft_ms_mean",
+                                         "tpot_ms_mean")}
+    log(f"{name}: workload {w['value']} generated tok/s, {w['all_tokens_per_s']} tok/s with the prompts")
+    return out
 
 
 def main():
@@ -320,17 +432,18 @@ def main():
     ap.add_argument("--no-check", action="store_true", help="profiling aid: skip the check before timing")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="profiling aid: run one of the two workloads (the JSON line then lacks the other)")
+    ap.add_argument("--quick", action="store_true",
+                    help="the headline alone: no decode at context 8,192, no 9B and 27B figures")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not measured")
         sys.exit(2)
     if a.workload:
-        return run_workload(a.workload, a)
+        print(json.dumps(run_workload(a.workload, a)), flush=True)
+        return
 
     from zse_amd.engine.loading import random_model
-    from zse_amd.engine.runner import StepEntry, StepRunner
     from zse_amd.runtime.device import Runtime
-    from zse_amd.sampling.sampler import DeviceSampler, SamplingParams
 
     cfg = dict(MODELS[a.model])
     full_layers = cfg["num_hidden_layers"]
@@ -360,121 +473,77 @@ def main():
     log(f"probes: {peak_bw / 1e9:.0f} GB/s streamed, {peak_fl / 1e12:.0f} TFLOP/s bf16 on the matrix cores")
 
     max_b = max(points)
-    page = 16
-    longest = max(a.context, a.prefill_tokens)       # a prompt longer than the decode context still fits
-    runner = StepRunner(model, rt, "bfloat16", page_size=page,
-                        num_pages=max(max_b * (-(-a.context // page) + 1), -(-longest // page)) + 8, max_seqs=max_b,
-                        max_batch_tokens=max(a.prefill_tokens, max_b), max_model_len=longest,
-                        use_graphs=not a.no_graphs)
-    sampler = DeviceSampler(rt, runner.k, max_b)
-    # Steady state is what is measured.  For about a second after a process has allocated tens of
-    # GB (the cache slabs, just now) kernels that wait for memory rather than stream from it run
-    # up to 17 % slower (the o and down products of a decode step: 10.1 instead of 8.7 us; steps
-    # at batch 1 and 8 by 3 to 4 %); later steps of the same process do not, whatever was done
-    # meanwhile.  So the timed work starts two seconds after the allocations.
-    rt.sync()
-    time.sleep(2.0)
-    greedy = SamplingParams(temperature=0.0)
-    rng = np.random.default_rng(0)
+    t = Timed(model, rt, cfg, max_b, a.context, a.prefill_tokens, not a.no_graphs)
+    runner = t.runner
     log(f"model ready in {time.time() - t0:.1f} s: {cfg['num_hidden_layers']} layers, "
         f"{model.weight_bytes / 1e9:.2f} GB of weights, cache {runner.cache_bytes() / 1e9:.2f} GB")
 
-    # ---- prefill: one prompt of 2,048 tokens in one step
+    # ---- prefill: one prompt of 2,048 tokens in one step, and the same prompt in portions of 512
     T = a.prefill_tokens
-    times = []
-    for i in range(4 if a.only != "decode" else 0):
-        toks = rng.integers(0, V, T).tolist()
-        rt.sync()
-        t1 = time.perf_counter()
-        runner.step([StepEntry(f"p{i}", toks, [T - 1])], download=False)
-        rt.sync()
-        times.append(time.perf_counter() - t1)
-        runner.finish(f"p{i}")
     prefill = None
-    if times:
-        pre_s = float(np.median(times[1:]))
-        pf = prefill_flops(cfg, T)
+    if a.only != "decode":
+        pre_s, pf = t.prefill()
         prefill = {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
                    "frac": round(pf / pre_s / PEAK_FLOPS["bf16"], 4), "frac_probed": round(pf / pre_s / peak_fl, 4)}
         log(f"prefill {T} tokens: {pre_s * 1e3:.2f} ms")
+        if T > 512:
+            ch_s, ch_f = t.prefill(portion=512)
+            prefill["chunked_512"] = {"value": round(T / ch_s, 1), "ms": round(ch_s * 1e3, 3), "steps": -(-T // 512),
+                                      "frac": round(ch_f / ch_s / PEAK_FLOPS["bf16"], 4)}
+            log(f"prefill {T} tokens in portions of 512: {ch_s * 1e3:.2f} ms")
     if a.only == "prefill":
         print(json.dumps({"prefill": prefill}), flush=True)
         return
 
     # ---- decode at each batch size, ending at the full context
-    def decode(B, steps, warmup):
-        ctx0 = a.context - steps - warmup
-        reqs = [f"d{B}_{i}" for i in range(B)]
-        for r in reqs:                       # fill the cache through real prefill steps
-            left = ctx0
-            while left > 0:
-                n = min(left, T)
-                runner.step([StepEntry(r, rng.integers(0, V, n).tolist(), [])], download=False)
-                left -= n
-        first = rng.integers(0, V, B).tolist()
-        rows = [{"params": greedy, "u": 0.0} for _ in range(B)]
-        # As the engine decodes: the sampling kernel leaves the ids on the device, the next step
-        # takes them from there, and the host reads them four steps at a time (it has to, for
-        # stop tokens) while the next steps are already enqueued.
-        sampler.prepare_run(rows, [[0.0] * B])
-        pending, fed = [], None
-
-        def one():
-            nonlocal fed
-            toks = first if fed is None else [0] * B
-            logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(reqs, toks)], download=False,
-                                 tokens_from=fed)
-            ids = sampler.sample_deferred(logits, 0)
-            fed = ids.device_ptr
-            pending.append(ids)
-            if len(pending) == 4:
-                for p in pending:
-                    p.result()
-                pending.clear()
-        for _ in range(warmup):
-            one()
-        rt.sync()
-        t1 = time.perf_counter()
-        for _ in range(steps):
-            one()
-        rt.sync()
-        dt = time.perf_counter() - t1
-        for r in reqs:
-            runner.finish(r)
-        mean_ctx = a.context - steps / 2.0
-        byts = weight_bytes(cfg) + B * cache_bytes(cfg, int(mean_ctx))
-        return B * steps / dt, dt / steps, byts
-
     results = {}
     for B in points:
         k = a.steps if B == a.batch else max(16, a.steps // 2)
         w = a.warmup if B == a.batch else max(4, a.warmup // 2)
-        results[B] = decode(B, k, w)
+        results[B] = t.decode(B, k, w)
         log(f"decode batch {B}: {results[B][0]:.1f} tok/s, {results[B][1] * 1e3:.3f} ms/step, "
-            f"{results[B][2] / results[B][1] / 1e9:.0f} GB/s")
+            f"{results[B][2] / results[B][1] / 1e9:.0f} GB/s ({results[B][3]})")
+    graph_max_batch = runner.graph_max_batch
+    t.close()
 
-    tok_s, step_s, byts = results[a.batch]
+    tok_s, step_s, byts, _ = results[a.batch]
     out = {
         "metric": "decode tok/s, Gemma 2 %s bf16, batch %d" % (a.model.upper(), a.batch),
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"model": f"gemma2-{a.model}-shapes-random", "layers": cfg["num_hidden_layers"],
-                   "layers_full": full_layers, "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
-                   "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
-                   "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
-                   "sliding_window": cfg["sliding_window"], "global_batch": a.batch, "seq_len": a.context,
-                   "prompt_len": a.prefill_tokens, "page_size": page, "parallelism": "single-gpu",
-                   "graphs": int(runner.use_graphs), "graph_max_batch": runner.graph_max_batch},
+        "config": dict(shape_of(cfg, full_layers), model=f"gemma2-{a.model}-shapes-random", global_batch=a.batch,
+                       seq_len=a.context, prompt_len=a.prefill_tokens, page_size=16, parallelism="single-gpu",
+                       graphs=int(not a.no_graphs), graph_max_batch=graph_max_batch),
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(byts / step_s / 1e9, 1), "peak": PEAK_HBM / 1e9,
                      "unit": "GB/s", "frac": round(byts / step_s / PEAK_HBM, 4),
                      "frac_probed": round(byts / step_s / peak_bw, 4)},
         "points": {f"decode_b{B}": round(results[B][0], 1) for B in points if B != a.batch},
         "points_roofline_frac": {f"decode_b{B}": round(results[B][2] / results[B][1] / PEAK_HBM, 4) for B in points},
+        "points_launched": {f"decode_b{B}": results[B][3] for B in points},
         "probed": {"hbm_gbs": round(peak_bw / 1e9, 1), "mfma_bf16_tflops": round(peak_fl / 1e12, 1)},
         "checked": check is not None, "check": check,
     }
+
+    # ---- further sizes: the same model at a context of 8,192 (the window then halves what the
+    # sliding layers read), and the 9B and 27B shapes with their workloads
+    if not a.quick and not a.only and a.model == "2b" and not a.layers:
+        t8 = Timed(model, rt, cfg, max_b, 8192, a.prefill_tokens, not a.no_graphs)
+        for B in points:
+            r = t8.decode(B, max(16, a.steps // 2), max(4, a.warmup // 2))
+            out["points"][f"decode_b{B}_ctx8192"] = round(r[0], 1)
+            out["points_roofline_frac"][f"decode_b{B}_ctx8192"] = round(r[2] / r[1] / PEAK_HBM, 4)
+            out["points_launched"][f"decode_b{B}_ctx8192"] = r[3]
+            log(f"decode batch {B} at context 8192: {r[0]:.1f} tok/s, {r[1] * 1e3:.3f} ms/step, {r[2] / r[1] / 1e9:.0f} GB/s")
+        t8.close()
+        del t8, t, runner, model
+        out["further"] = {}
+        for name in ("9b", "27b"):
+            out["further"][name] = further_model(name, a, rt, peak_bw, peak_fl)
+            out["points"][f"{name}_decode_b8"] = out["further"][name]["decode_b8"]["value"]
+            out["points"][f"{name}_prefill_2048"] = out["further"][name]["prefill"]["value"]
+            out["points"][f"{name}_workload"] = out["further"][name]["workload"]["value"]
     print(json.dumps(out), flush=True)
 
 

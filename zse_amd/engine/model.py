@@ -66,6 +66,37 @@ class Model:
                 out.append(self.blocks[call.layer].mixer.cache_need())
         return out
 
+    # ---- what a step costs, for measurements: read off the parts, whatever the architecture
+    def flops(self, portions, rows: int) -> float:
+        """Flops of a step: ``portions`` is a list of (start, n) with n tokens of a request
+        behind ``start`` cached ones, ``rows`` the number of logit rows asked for."""
+        tokens = sum(n for _, n in portions)
+        total = 0.0
+        for call in self.plan.order:
+            blk = self.blocks[call.layer]
+            total += tokens * sum(p.flops_per_token() for p in walk(blk))
+            mixer = getattr(blk, "mixer", None)
+            need = mixer.cache_need() if mixer is not None else None
+            if isinstance(need, PagedKV):
+                for start, n in portions:
+                    last = start + n          # keys the portion's last token sees, without a window
+                    if need.window and last > need.window:
+                        full = max(0, min(n, last - need.window))          # tokens that see a whole window
+                        keys = full * need.window + sum(range(last - n + 1, last - full + 1))
+                    else:
+                        keys = sum(range(start + 1, last + 1))
+                    total += mixer.flops_per_key() * keys
+        return total + rows * self.head.flops_per_token()
+
+    def cache_bytes_read(self, context: int, itemsize: int) -> int:
+        """Bytes of cached keys and values that one token at position ``context - 1`` reads."""
+        total = 0
+        for need in self.cache_needs():
+            if isinstance(need, PagedKV):
+                seen = min(context, need.window) if need.window else context
+                total += 2 * need.num_kv_heads * need.head_dim * seen * itemsize
+        return total
+
     def forward(self, ctx, caches: List[CallCache], logit_rows, n_rows: int, logits: Tensor):
         """Run the step's tokens through every entry of the order; write float
         logits of the rows ``logit_rows`` (device int32 pointer) into ``logits``."""

@@ -59,6 +59,9 @@ class PagedAttention(Part):
         s = self.spec
         return PagedKV(s.num_kv_heads, s.head_dim, s.window)
 
+    def flops_per_key(self) -> float:
+        return 4.0 * self.spec.num_heads * self.spec.head_dim        # q.k and p.v
+
     PORTION_RANGES_BYTES = 192 << 20
 
     def wants_v_transposed(self, kernels, dtype: str, page_size: int) -> bool:

@@ -68,6 +68,18 @@ class Part:
     def children(self) -> List["Part"]:
         return []
 
+    def flops_per_token(self) -> float:
+        """Multiply-adds x 2 that one token costs in this part's own matrices (children not
+        counted): what measurements price a step with.  The default reads it off the matrices
+        the part asks for; a part that uses only some of them for a token (routed experts), or
+        none (a table that is gathered from), says so itself."""
+        return float(sum(2 * r.shape[0] * r.shape[1] for r in self.tensor_reqs()
+                         if r.role == ROLE_MATRIX and len(r.shape) == 2))
+
+    def flops_per_key(self) -> float:
+        """A mixer over cached keys: multiply-adds x 2 per (token, key it attends to)."""
+        return 0.0
+
     def prepare(self, kernels, dtype: str, max_seqs: int, max_model_len: int, page_size: int,
                 max_batch_tokens: int = 0) -> int:
         """Called once by the step runner, with its limits, before the first step.  A part

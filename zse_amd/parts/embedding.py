@@ -42,6 +42,9 @@ class Embedding(Part):
             s = bf16_bits_to_f32(f32_to_bf16_bits(np.array([s])))[0]
         self.scale = float(s)
 
+    def flops_per_token(self) -> float:
+        return 0.0           # rows are gathered, not multiplied
+
     def forward(self, ctx) -> Tensor:
         s = self.spec
         h = ctx.alloc((ctx.T, s.hidden_size), F32)
