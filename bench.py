@@ -177,9 +177,9 @@ def check_decode_path(model, rt, vocab, B, use_graphs):
             fed, pending = None, []
             for _ in range(n_steps):
                 toks = ids[0] if fed is None else [0] * B
-                logits = runner.step([StepEntry(i, [t], [0]) for i, t in enumerate(toks)], download=False,
-                                     tokens_from=fed)
-                pending.append(sampler.sample_deferred(logits, 0))
+                chosen = runner.step([StepEntry(i, [t], [0]) for i, t in enumerate(toks)], download=False,
+                                     tokens_from=fed, pick=True)
+                pending.append(sampler.ids_deferred(chosen))
                 fed = pending[-1].device_ptr
             ids += [list(p.result()) for p in pending]
             if use_graphs and B <= runner.graph_max_batch and not any(isinstance(g, int) for g in runner.graphs.values()):
@@ -262,6 +262,7 @@ def run_workload(name, a, model=None):
         "workload": what, "seconds": round(dt, 3), "generated_tokens": gen, "prompt_tokens": prompt_tokens,
         "all_tokens_per_s": round((gen + prompt_tokens) / dt, 1), "steps": st.steps - steps0,
         "preemptions": st.preemptions,
+        "launched": {"graph": st.graph_steps, "launch_list": st.launch_list_steps, "python": st.python_steps},
         "config": {"model": f"gemma2-{name}-shapes-random", "layers": cfg["num_hidden_layers"], "layers_full": full_layers,
                    "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
@@ -341,18 +342,18 @@ class Timed:
                 left -= n
         first = rng.integers(0, V, B).tolist()
         rows = [{"params": SamplingParams(temperature=0.0), "u": 0.0} for _ in range(B)]
-        # As the engine decodes: the sampling kernel leaves the ids on the device, the next step
-        # takes them from there, and the host reads them four steps at a time (it has to, for
-        # stop tokens) while the next steps are already enqueued.
+        # As the engine decodes greedily: the step picks the largest logits itself and leaves the
+        # ids on the device, the next step takes them from there, and the host reads them four
+        # steps at a time (it has to, for stop tokens) while the next steps are already enqueued.
         sampler.prepare_run(rows, [[0.0] * B])
         pending, fed = [], None
 
         def one():
             nonlocal fed
             toks = first if fed is None else [0] * B
-            logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(reqs, toks)], download=False,
-                                 tokens_from=fed)
-            ids = sampler.sample_deferred(logits, 0)
+            picked = runner.step([StepEntry(r, [t], [0]) for r, t in zip(reqs, toks)], download=False,
+                                 tokens_from=fed, pick=True)
+            ids = sampler.ids_deferred(picked)
             fed = ids.device_ptr
             pending.append(ids)
             if len(pending) == 4:
@@ -408,7 +409,7 @@ def further_model(name, a, rt, peak_bw, peak_fl):
         f"prefill {pre_s * 1e3:.2f} ms ({out['prefill']['frac']} of 2.5 PFLOP/s)")
     w = run_workload(name, a, model=model)
     out["workload"] = {k: w[k] for k in ("value", "unit", "workload", "seconds", "generated_tokens", "prompt_tokens",
-                                         "all_tokens_per_s", "steps", "preemptions", "by_kind", "ttft_ms_mean",
+                                         "all_tokens_per_s", "steps", "preemptions", "launched", "by_kind", "ttft_ms_mean",
                                          "tpot_ms_mean")}
     log(f"{name}: workload {w['value']} generated tok/s, {w['all_tokens_per_s']} tok/s with the prompts")
     return out

@@ -1006,6 +1006,63 @@ def test_lm_head_product_at_full_vocabulary(rt):
         assert np.all(got.std(axis=0) > 0) if M >= 8 else np.count_nonzero(got) > N * 0.99
 
 
+def test_the_head_that_picks_without_writing_logits(rt):
+    """zk_head_pick_bf16 against the product with the soft cap followed by zk_argmax, on the
+    full vocabulary of 256,000 (and one that is no whole number of strips), 1 to 64 rows, with
+    ties: rows of W that are copies of each other (equal logits: the lower column wins), and
+    activations so large that the cap saturates and hundreds of columns hold the same largest
+    value.  The same ids, bit for bit; nothing but the ids and the strips' picks is written."""
+    k = rt.kernels("bfloat16")
+    K, cap = 2304, 30.0
+    rng = np.random.default_rng(11)
+    for N in (256000, 4999):
+        w = bf16(rng.normal(size=(N, K)) * 0.05)
+        for a, b in ((17, 3), (N - 1, 4000), (N // 2 + 5, N // 2 + 4)):       # copies: later columns equal earlier ones
+            w[a] = w[b]
+        W = up(rt, w, "bfloat16")
+        rows = (N + 15) // 16 * 16
+        Ws = rt.zeros((rows, K), "bfloat16")
+        k.zk_strip_layout(W.ptr, Ws.ptr, N, K, rt.stream)
+        ws = gemm_workspace(rt)
+        for M in (1, 8, 16, 24, 64):
+            a = rng.normal(size=(M, K))
+            a[0] = w[3] * 40                           # row 0 points at column 3 and its copy, column 17
+            if M > 1:
+                a[M - 1] = w[4000 % N] * 40
+            if M > 2:
+                a[1] *= 100                            # far beyond the cap: many columns saturate at 30.0
+            a = bf16(a)
+            A = up(rt, a, "bfloat16")
+            logits = rt.zeros((M, N), "float32")
+            k.zk_gemm_bf16(A.ptr, K, Ws.ptr, logits.ptr, N, 1, M, N, K, 1, cap, 1, ws.ptr, ws.nbytes, None, rt.stream)
+            want = rt.zeros((M,), "int32")
+            scratch = rt.zeros((M * 64 * 2,), "float32")
+            k.zk_argmax(logits.ptr, want.ptr, M, N, scratch.ptr, rt.stream)
+            picks = rt.zeros((k.zk_head_pick_bf16_workspace(M, N) // 4 + 4,), "float32")
+            got = rt.zeros((M,), "int32")
+            k.zk_head_pick_bf16(A.ptr, K, Ws.ptr, M, N, K, cap, 1, picks.ptr, picks.nbytes, got.ptr, rt.stream)
+            want, got, z = rt.download(want), rt.download(got), rt.download(logits)
+            assert np.array_equal(got, want), (N, M, got, want)
+            assert np.array_equal(want, z.argmax(axis=1))             # NumPy's argmax keeps the first maximum too
+            assert want[0] == 3 and (z[0, 17] == z[0, 3])
+            if M > 2:
+                assert np.count_nonzero(z[1] == z[1].max()) > 50, "the cap was meant to saturate"
+        # row-major weights (no strip layout) serve up to 16 rows
+        A = up(rt, bf16(rng.normal(size=(5, K))), "bfloat16")
+        logits, want, got = rt.zeros((5, N), "float32"), rt.zeros((5,), "int32"), rt.zeros((5,), "int32")
+        k.zk_gemm_bf16(A.ptr, K, W.ptr, logits.ptr, N, 1, 5, N, K, 1, cap, 0, ws.ptr, ws.nbytes, None, rt.stream)
+        scratch = rt.zeros((5 * 64 * 2,), "float32")
+        k.zk_argmax(logits.ptr, want.ptr, 5, N, scratch.ptr, rt.stream)
+        picks = rt.zeros((k.zk_head_pick_bf16_workspace(5, N) // 4 + 4,), "float32")
+        k.zk_head_pick_bf16(A.ptr, K, W.ptr, 5, N, K, cap, 0, picks.ptr, picks.nbytes, got.ptr, rt.stream)
+        assert np.array_equal(rt.download(got), rt.download(want))
+    from zse_amd.runtime.device import DeviceError
+    with pytest.raises(DeviceError, match="1 to 64 rows"):
+        k.zk_head_pick_bf16(A.ptr, K, Ws.ptr, 65, N, K, cap, 1, picks.ptr, picks.nbytes, got.ptr, rt.stream)
+    with pytest.raises(DeviceError, match="scratch too small"):
+        k.zk_head_pick_bf16(A.ptr, K, Ws.ptr, 5, N, K, cap, 1, picks.ptr, 64, got.ptr, rt.stream)
+
+
 # ------------------------------------------------------------------ random weights
 @pytest.mark.parametrize("n", [1, 2, 7, 4096, 1_000_003])
 def test_device_random_weights_equal_the_host_function_bit_for_bit(rt, n):

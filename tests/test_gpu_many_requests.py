@@ -157,9 +157,26 @@ def test_the_engine_with_24_and_64_places(tiny_folders, name, seqs, dtype):
     st = eng.stats()
     assert most > 16 and most >= seqs * 5 // 8, most
     assert st.preemptions > 0, "the pool was meant to be too small"
-    if all(sp.temperature == 0.0 for sp in params):
-        assert eng.runner.steplist_runs > 0, "no decode step of more than 16 requests ran from its list"
     assert all(pool.free_pages == pool.num_pages for pool in eng.runner.manager.pools)
+    # and a full house in lockstep: as many short prompts as there are places, all admitted in one
+    # step, all greedy, all as long: every decode step brings one token of each, more than a
+    # graph takes, so runs of four steps are launched from one written-down list, the ids fed
+    # from step to step on the device
+    lists0 = eng.runner.steplist_runs
+    short = [random_tokens(V, 3, 9000 + i) for i in range(seqs)]
+    together = eng.generate(short, SamplingParams(max_tokens=10, temperature=0.0))
+    assert eng.runner.steplist_runs - lists0 >= 6, "decode steps of a full house did not run from their list"
+    eng.close()
+    eng = engine(1, 64, 1)
+    for p, got in list(zip(short, together))[::5]:
+        a = eng.generate([p], SamplingParams(max_tokens=10, temperature=0.0))[0]
+        if dtype == "float32":
+            assert got == a
+        else:
+            same_upto = next((j for j in range(10) if a[j] != got[j]), 10)
+            if same_upto < 10:
+                z = np.sort(P.forward(cfg, w, list(p) + got[:same_upto], np.float64)[-1])
+                assert z[-1] - z[-2] < 0.05
     eng.close()
 
     same = 0

@@ -275,8 +275,8 @@ def test_a_part_brings_a_kernel_of_its_own(rt, dtype):
     streams = {"a": rng.integers(0, V, 29).tolist(), "b": rng.integers(0, V, 17).tolist()}
     # portions of sizes that come back, then single tokens side by side: shapes repeat, so launch
     # lists run and the graph of bucket 2 is captured and replayed
-    steps = [[("a", 5)], [("b", 5)], [("a", 5), ("b", 3)], [("a", 5), ("b", 3)], [("a", 2)], [("b", 2)]]
-    steps += [[("a", 1), ("b", 1)] for _ in range(4)] + [[("a", 1)] for _ in range(8)]
+    steps = [[("a", 5)], [("b", 5)], [("a", 5)], [("b", 5)], [("a", 5)], [("b", 2)]]
+    steps += [[("a", 1), ("b", 1)] for _ in range(4)] + [[("b", 1)]] + [[("a", 1)] for _ in range(10)]
 
     def run(runner):
         fed = {r: 0 for r in streams}

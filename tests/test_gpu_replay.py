@@ -452,7 +452,8 @@ def test_steps_launched_from_their_written_down_lists(cases, dtype):
     plain_rows, plain_runner = run(False)
     listed_rows, runner = run(True)
     assert plain_runner.steplist_runs == 0 and not plain_runner.steplists
-    assert runner.use_steplists and runner.steplist_runs >= 12 and 0 < len(runner.steplists) <= 8
+    assert runner.use_steplists and runner.steplist_runs >= 11 and 0 < len(runner.steplists) <= 8
+    assert runner.steplist_runs + runner.steplist_misses == len(steps)
     assert all(runner.k.steplist_size(h) > 10 for h in runner.steplists.values())
     for r in reqs:
         assert np.array_equal(listed_rows[r], plain_rows[r]), r

@@ -48,7 +48,44 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-enum { EPI_NONE = 0, EPI_SOFTCAP = 1, EPI_GELU_TANH = 2, EPI_SILU = 3 };
+// EPI_PICK (the LM head of a step whose next tokens are the largest logits): nothing of C is
+// stored; each strip of 16 columns leaves, per row, its largest value after the soft cap (cap
+// <= 0: none) and that value's column in ``partials`` [M][strips] as (float, int), larger value
+// first, equal values to the lower column, NaN never, which a joining kernel reduces to one
+// column a row: the greedy choice without the logits ever reaching memory.
+enum { EPI_NONE = 0, EPI_SOFTCAP = 1, EPI_GELU_TANH = 2, EPI_SILU = 3, EPI_PICK = 4 };
+
+struct Pick {
+  float value;
+  int column;
+};
+
+// A lane's four results x[i] at columns n + i of one row, joined with the lanes 16, 32 and 48
+// further on (the other columns of the strip); afterwards every one of the four lanes holds
+// the strip's pick.
+__device__ __forceinline__ Pick pick_of_strip(const float (&x)[4], int n, int N, float cap) {
+  Pick p{-INFINITY, 0x7fffffff};
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    if (n + i >= N) continue;
+    const float v = cap > 0.f ? cap * tanhf(x[i] / cap) : x[i];
+    if (v > p.value || (p.column == 0x7fffffff && v == v)) {
+      p.value = v;
+      p.column = n + i;
+    }
+  }
+#pragma unroll
+  for (int off = 16; off <= 32; off *= 2) {
+    const float ov = __shfl_xor(p.value, off);
+    const int oc = __shfl_xor(p.column, off);
+    const bool other_valid = oc != 0x7fffffff, mine_valid = p.column != 0x7fffffff;
+    if (other_valid && (!mine_valid || ov > p.value || (ov == p.value && oc < p.column))) {
+      p.value = ov;
+      p.column = oc;
+    }
+  }
+  return p;
+}
 
 // 0.5 g (1 + tanh(u)) = g / (1 + exp(-2 u)): one exponential and one reciprocal instead of the
 // library's tanh, which cost a tenth of the prompt's gate|up product; the difference (a few
@@ -323,6 +360,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
 #pragma unroll
         for (int i = 0; i < 4; i++) vt[(size_t)(at + i) * rs.bs] = (__bf16)x[i];
       }
+      continue;
+    }
+    if (!GATED && epi == EPI_PICK) {
+      const float x[4] = {v[0][0], v[0][1], v[0][2], v[0][3]};
+      const Pick p = pick_of_strip(x, n0 + 4 * kq, N, cap);
+      if (kq == 0 && m < M) ((Pick*)partials)[(size_t)m * gridDim.x + blockIdx.x] = p;
       continue;
     }
     if (m >= M) continue;
@@ -922,11 +965,18 @@ static bool joinable_by_reader(int N, int ldc, int c_is_f32, int epi) {
 // A lane's results of one strip: rows n = 16 * strip + 4 * kq + i of W, column m = 16 * mt + r of A.
 template <int MT, bool GATED>
 __device__ __forceinline__ void mid_store(const f32x4 (&acc)[GATED ? 2 : 1][MT], void* __restrict__ C, int ldc,
-                                          int c_is_f32, int M, int N, int strip, int lane, int epi, float cap) {
+                                          int c_is_f32, int M, int N, int strip, int lane, int epi, float cap,
+                                          float* __restrict__ picks, int nstrips) {
   const int r = lane & 15, kq = lane >> 4;
 #pragma unroll
   for (int mt = 0; mt < MT; mt++) {
     const int m = mt * 16 + r;
+    if (!GATED && epi == EPI_PICK) {
+      const float x[4] = {acc[0][mt][0], acc[0][mt][1], acc[0][mt][2], acc[0][mt][3]};
+      const Pick p = pick_of_strip(x, strip * 16 + 4 * kq, N, cap);
+      if (kq == 0 && m < M) ((Pick*)picks)[(size_t)m * nstrips + strip] = p;
+      continue;
+    }
     if (m >= M) continue;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -1077,7 +1127,7 @@ __global__ __launch_bounds__(512) void gemm_mid_kernel(const __bf16* __restrict_
         if (mt * 16 + r < M) *(f32x4*)(planes + ((size_t)g * M + mt * 16 + r) * npad) = acc[g][mt];
     return;
   }
-  if (strip_ok) mid_store<MT, GATED>(acc, C, ldc, c_is_f32, M, N, strip, lane, epi, cap);
+  if (strip_ok) mid_store<MT, GATED>(acc, C, ldc, c_is_f32, M, N, strip, lane, epi, cap, partials, nstrips);
 }
 
 // Second half of a mid product whose K was split over blocks: `ksplit`
@@ -1144,7 +1194,7 @@ static int launch_mid(const void* A, int lda, const void* W, void* C, int ldc, i
   }
   const size_t per_range = (size_t)(GATED ? 2 : 1) * M * npad * sizeof(float);
   void* ws = wsp.ptr;
-  if (ws == nullptr || (uintptr_t)ws % 16 != 0) ksplit = 1;
+  if (ws == nullptr || (uintptr_t)ws % 16 != 0 || epi == EPI_PICK) ksplit = 1;      // picks are taken from whole sums
   while (ksplit > 1 && ksplit * per_range > wsp.split_bytes()) ksplit--;
   if (ksplit > 1 && ksplit * per_range > wsp.bytes) return wsp.too_small(ksplit * per_range);
   float* partials = (float*)ws;
@@ -1209,10 +1259,12 @@ static int launch_skinny(const void* A, int lda, const void* W, void* C, int ldc
   do {                                                                                                \
     if (w_strip)                                                                                      \
       gemm_skinny_kernel<MT_, GATED, NW_, false, true><<<grid, NW_ * 64, 0, s>>>(                     \
-          (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, RopeStore{}); \
+          (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, RopeStore{}, \
+          partials, 1);                                                                               \
     else                                                                                              \
       gemm_skinny_kernel<MT_, GATED, NW_><<<grid, NW_ * 64, 0, s>>>(                                  \
-          (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, RopeStore{}); \
+          (const __bf16*)A, lda, (const __bf16*)W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, RopeStore{}, \
+          partials, 1);                                                                               \
   } while (0)
   if (ksplit > 1) {
     if constexpr (!GATED) {
@@ -1370,10 +1422,10 @@ static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc
   ZK_REQUIRE(M >= 0 && N > 0 && K > 0, "zk_gemm_bf16: bad sizes");
   ZK_REQUIRE(K % 8 == 0 && lda % 8 == 0, "zk_gemm_bf16: K and lda must be multiples of 8");
   ZK_REQUIRE(lda >= K && ldc >= N, "zk_gemm_bf16: leading dimensions too small");
-  ZK_REQUIRE(epi >= 0 && epi <= 3, "zk_gemm_bf16: unknown epilogue");
+  ZK_REQUIRE(epi >= 0 && epi <= EPI_PICK, "zk_gemm_bf16: unknown epilogue");
   ZK_REQUIRE(epi != EPI_SOFTCAP || cap > 0.f, "zk_gemm_bf16: soft cap must be positive");
   ZK_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "zk_gemm_bf16: operands must be 16-byte aligned");
-  const bool gated = epi >= EPI_GELU_TANH;
+  const bool gated = epi == EPI_GELU_TANH || epi == EPI_SILU;
   ZK_REQUIRE(!w_strip || (K % 32 == 0 && (!gated || N % 16 == 0)), "zk_gemm_bf16: strip layout needs K % 32 == 0 (and N % 16 == 0 when gated)");
   if (parts) *parts = 0;
   if (M == 0) return 0;
@@ -1479,8 +1531,74 @@ static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc
 extern "C" int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32,
                             int M, int N, int K, int epi, float cap, int w_strip, void* ws,
                             size_t ws_bytes, int* parts, void* stream) {
+  ZK_REQUIRE(epi != EPI_PICK, "zk_gemm_bf16: the picking epilogue belongs to zk_head_pick_bf16");
   return gemm_bf16_run(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip, GemmWorkspace{ws, ws_bytes, false},
                        parts, stream);
+}
+
+// ---- the LM head of a greedy step: the largest logit's column of every row, no logits stored
+//
+// One block a row joins the strips' picks: larger value first, equal values to the lower
+// column, NaN never; a row without any valid value gets column 0 (as zk_argmax does).
+__global__ __launch_bounds__(1024) void pick_join_kernel(const Pick* __restrict__ picks, int nstrips,
+                                                         int* __restrict__ ids) {
+  __shared__ float sv[16];
+  __shared__ int sc[16];
+  const Pick* row = picks + (size_t)blockIdx.x * nstrips;
+  Pick best{-INFINITY, 0x7fffffff};
+  auto better = [](const Pick& a, const Pick& b) {       // a before b
+    if (a.column == 0x7fffffff) return false;
+    return b.column == 0x7fffffff || a.value > b.value || (a.value == b.value && a.column < b.column);
+  };
+  // eight loads of a thread on their way at a time (a place past the end reads the last pick
+  // again, which changes nothing): with one block a row the time is the trips to memory
+  for (int i0 = threadIdx.x; i0 < nstrips; i0 += 8 * 1024) {
+    Pick p[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) p[j] = row[min(i0 + j * 1024, nstrips - 1)];
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+      if (better(p[j], best)) best = p[j];
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const Pick o{__shfl_xor(best.value, off), __shfl_xor(best.column, off)};
+    if (better(o, best)) best = o;
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) {
+    sv[wave] = best.value;
+    sc[wave] = best.column;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 16; w++) {
+      const Pick o{sv[w], sc[w]};
+      if (better(o, best)) best = o;
+    }
+    ids[blockIdx.x] = best.column == 0x7fffffff ? 0 : best.column;
+  }
+}
+
+extern "C" size_t zk_head_pick_bf16_workspace(int M, int N) {
+  return (size_t)(M > 0 ? M : 0) * (size_t)((N + 15) / 16) * sizeof(Pick);
+}
+
+// ids[m] = the column of the largest value of row m of A W^T after the soft cap (cap <= 0: no
+// cap): what zk_gemm_bf16 with the soft-cap epilogue followed by zk_argmax gives, bit for bit,
+// without the [M, N] logits.  1 to 64 rows; more than 16 need W in strip layout.  ``picks``:
+// zk_head_pick_bf16_workspace(M, N) bytes of scratch, 16-byte aligned.
+extern "C" int zk_head_pick_bf16(const void* A, int lda, const void* W, int M, int N, int K, float cap, int w_strip,
+                                 void* picks, size_t picks_bytes, void* ids, void* stream) {
+  ZK_REQUIRE(M >= 1 && M <= 64, "zk_head_pick_bf16: 1 to 64 rows");
+  ZK_REQUIRE(M <= 16 || w_strip, "zk_head_pick_bf16: more than 16 rows need the weights in strip layout");
+  ZK_REQUIRE(picks != nullptr && (uintptr_t)picks % 16 == 0 && ids != nullptr, "zk_head_pick_bf16: no scratch or no result");
+  ZK_REQUIRE(picks_bytes >= zk_head_pick_bf16_workspace(M, N), "zk_head_pick_bf16: scratch too small");
+  if (int rc = gemm_bf16_run(A, lda, W, nullptr, N, 1, M, N, K, EPI_PICK, cap, w_strip,
+                             GemmWorkspace{picks, picks_bytes, false}, nullptr, stream))
+    return rc;
+  pick_join_kernel<<<M, 1024, 0, (hipStream_t)stream>>>((const Pick*)picks, (N + 15) / 16, (int*)ids);
+  return zk_launch_status("zk_head_pick_bf16");
 }
 
 // ---- the same product for callers that cannot allocate (declared in gemm_bf16_static.h)
@@ -1529,6 +1647,7 @@ extern "C" int zk_gemm_bf16_static(const void* A, int lda, const void* W, void* 
   // results have the same bits; a split whose partial sums do not fit the array is refused.
   // Nothing in the array has to start at zero: each range's plane is written in full by the
   // product kernel before the joining kernel of the same call reads it.
+  ZK_REQUIRE(epi != EPI_PICK, "zk_gemm_bf16_static: the picking epilogue belongs to zk_head_pick_bf16");
   return gemm_bf16_run(A, lda, W, C, ldc, c_is_f32, M, N, K, epi, cap, w_strip,
                        GemmWorkspace{ptr, ZK_GEMM_STATIC_SCRATCH_BYTES, true}, nullptr, stream);
 }

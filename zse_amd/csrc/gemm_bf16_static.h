@@ -9,8 +9,11 @@
 //
 //  * The array holds ZK_GEMM_STATIC_SCRATCH_BYTES on every GPU the library runs on, from the
 //    library's first use on that GPU until the process ends.
-//  * K is split exactly as zk_gemm_bf16 splits it with its standard workspace
-//    (zk_gemm_bf16_workspace() bytes), so both give the same bits.  A shape whose partial sums
+//  * K is split exactly as zk_gemm_bf16 splits it when it is called with its standard workspace
+//    (zk_gemm_bf16_workspace() bytes) and without ``parts``, so both give the same bits.  (With
+//    ``parts`` a reader takes the partial sums over, and zk_gemm_bf16 may then split products
+//    of up to 16 rows that it otherwise leaves whole; this entry point has no such reader.)
+//    A shape whose partial sums
 //    do not fit the array is refused with an error that names both sizes; nothing is launched.
 //    Products of up to 64 rows always fit (their ranges times their padded width stay within
 //    32768 columns: 64 x 32768 floats, twice that with a gate, are the array's 16 MiB);

@@ -48,6 +48,8 @@ int zk_gemm_bf16(const void* A, int lda, const void* W, void* C, int ldc, int c_
 int zk_qkv_rope_bf16(const void* A, int lda, const void* W, void* Q, int ldq, int M, int K, int w_strip,
                      const int* positions, const int* slot_map, const float* inv_freq, void* kcache, void* vcache,
                      int nh, int nkv, int hd, int bs, int v_transposed, void* stream);
+int zk_head_pick_bf16(const void* A, int lda, const void* W, int M, int N, int K, float cap, int w_strip,
+                      void* picks, size_t picks_bytes, void* ids, void* stream);
 int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const void* vcache_t, const int* block_table,
                       int max_blocks, const int* q_start, const int* ctx_len, void* out, int R, int r_prefill,
                       int max_q_len, int max_ctx, int nh, int nkv, int hd, int bs, float scale, float softcap,
@@ -125,6 +127,7 @@ const int entered_at_load = []() {
   OWN(zk_gemm_bf16);
   OWN(zk_qkv_rope_bf16);
   OWN(zk_attention_bf16);
+  OWN(zk_head_pick_bf16);
 #endif
   return 0;
 }();

@@ -37,6 +37,12 @@ class EngineStats:
     # per finished request, with the reference's meanings (zstreamer/request.py:206-228)
     ttft_ms: List[float] = field(default_factory=list)
     tpot_ms: List[float] = field(default_factory=list)
+    # how the steps were launched: replayed from a captured graph, from a written-down launch
+    # list, or call by call from Python (a shape's first two steps, and every step of a model
+    # with a part that cannot be written down)
+    graph_steps: int = 0
+    launch_list_steps: int = 0
+    python_steps: int = 0
 
     @property
     def tokens_per_second(self) -> float:
@@ -202,8 +208,13 @@ class Engine:
             known = tokens_from is None
             entries = [StepEntry(r.request_id, [r.tokens_at(s.start, 1)[0] if known else 0], [0])
                        for r, s in zip(reqs, plan.items)]
-            logits = runner.step(entries, download=False, tokens_from=tokens_from)
-            ids = sampler.sample_deferred(logits, i)
+            if sampler.run_is_greedy:
+                # the step picks the largest logits itself (in the head product's epilogue where
+                # the kernels can: the logits then never reach memory)
+                ids = sampler.ids_deferred(runner.step(entries, download=False, tokens_from=tokens_from, pick=True))
+            else:
+                logits = runner.step(entries, download=False, tokens_from=tokens_from)
+                ids = sampler.sample_deferred(logits, i)
             pending.append(ids)
             tokens_from = ids.device_ptr
             done += sch.on_step_done(plan, {r.request_id: None for r in reqs})
@@ -290,10 +301,15 @@ class Engine:
             raise RuntimeError(f"request {req.request_id}: {req.error}")
 
     def stats(self) -> EngineStats:
-        return self._stats
+        if self.runner is not None:
+            self._launch_counts = (self.runner.graph_runs, self.runner.steplist_runs, self.runner.steplist_misses)
+        st = self._stats
+        st.graph_steps, st.launch_list_steps, st.python_steps = getattr(self, "_launch_counts", (0, 0, 0))
+        return st
 
     def close(self) -> None:
         if self.runner is not None:
+            self.stats()                       # keeps the runner's launch counts
             self.runner.close()
         self.runner = None
         self.sampler = None

@@ -97,9 +97,11 @@ class Model:
                 total += 2 * need.num_kv_heads * need.head_dim * seen * itemsize
         return total
 
-    def forward(self, ctx, caches: List[CallCache], logit_rows, n_rows: int, logits: Tensor):
+    def forward(self, ctx, caches: List[CallCache], logit_rows, n_rows: int, logits: Tensor, pick=None):
         """Run the step's tokens through every entry of the order; write float
-        logits of the rows ``logit_rows`` (device int32 pointer) into ``logits``."""
+        logits of the rows ``logit_rows`` (device int32 pointer) into ``logits``.
+        ``pick``: (ids, scratch) instead, for a step that wants nothing but each row's largest
+        logit's column and whose head can give it without writing the logits (``head.can_pick``)."""
         h = self.embedding.forward(ctx)
         order = self.plan.order
         # the norm that opens a layer is computed by the kernel that closes the one before;
@@ -121,5 +123,7 @@ class Model:
             ctx.arena.release(base)
         if n_rows:
             x = self.final_norm.forward(ctx, h, out_rows=(logit_rows, n_rows))
+            if pick is not None:
+                return self.head.pick(ctx, x, pick[0], pick[1])
             self.head.forward(ctx, x, logits)
         return logits

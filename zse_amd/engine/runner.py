@@ -253,10 +253,18 @@ class StepRunner:
         # are launched from there with one call (zk_steplist_run).  The same condition as for
         # graphs: what differs between steps of one shape must come from device memory.
         self.use_steplists = bool(use_steplists) and self.graph_safe
-        self.steplists: Dict[tuple, int] = {}        # shape of a step -> handle of its launch list
-        self.steplist_runs = 0
+        self.steplists: Dict[tuple, int] = {}        # shape of a step -> handle of its launch list, least recently used first
+        self._sighted: Dict[tuple, None] = {}        # shapes met once and not written down yet
+        self.steplist_runs = 0                       # eager steps launched from a list
+        self.steplist_misses = 0                     # eager steps launched call by call from Python
+        self.graph_runs = 0                          # decode steps replayed from a captured graph
         self.graph_logits: Optional[Tensor] = None
         self.steps_run = 0
+        # a step that wants nothing but each row's largest logit's column (``step(pick=True)``):
+        # the ids' buffer and the scratch memory of the head's picking product, made on first use
+        self.pick_ids: Optional[Tensor] = None
+        self.pick_scratch: Optional[Tensor] = None
+        self._head_picks: Dict[int, bool] = {}       # rows -> whether the head picks for that many
 
     # ------------------------------------------------------------------ sizes
     def _meta_words(self, T: int, R: int, G: int) -> int:
@@ -403,6 +411,29 @@ class StepRunner:
             self.logits = None
             self.logits = self.rt.empty((max(rows, 8), self.vocab), F32)
 
+    # ------------------------------------------------------------------ picking instead of logits
+    def _pick_buffers(self, rows: int):
+        """(ids, scratch) if the model's head picks for ``rows`` rows without writing logits,
+        else None (the step then writes logits and the argmax kernel reads them)."""
+        head = self.model.head
+        if self.pick_ids is None:
+            self.pick_ids = self.rt.empty((max(self.max_seqs, 8),), I32)
+            self.argmax_scratch = self.rt.empty((max(self.max_seqs, 8) * 64 * 2,), F32)
+        if not hasattr(head, "can_pick") or rows > self.pick_ids.shape[0]:
+            return None
+        if rows not in self._head_picks:
+            self._head_picks[rows] = bool(head.can_pick(StepContext(self), rows))
+        if not self._head_picks[rows]:
+            return None
+        if self.pick_scratch is None:
+            most = min(self.pick_ids.shape[0], head.PICK_ROWS)
+            self.pick_scratch = self.rt.empty(((head.pick_scratch_bytes(self.k, most) + 3) // 4,), F32)
+        return (self.pick_ids, self.pick_scratch)
+
+    def _argmax_of(self, logits: Tensor, n_rows: int) -> Tensor:
+        self.k.zk_argmax(logits.ptr, self.pick_ids.ptr, n_rows, self.vocab, self.argmax_scratch.ptr, self.rt.stream)
+        return self.pick_ids.rows(0, n_rows)
+
     # ------------------------------------------------------------------ graphs for decode steps
     def _graph_bucket(self, entries) -> int:
         """The padded batch size under which a decode-only step replays a captured graph
@@ -418,7 +449,7 @@ class StepRunner:
             b *= 2
         return b if b <= self.max_seqs else 0
 
-    def _graph_step(self, entries, bucket: int, tokens_from=None):
+    def _graph_step(self, entries, bucket: int, tokens_from=None, pick=False):
         """One token for each request through a graph of this bucket.  The first step of
         a bucket runs eagerly (it sizes the arena), later ones are captured and replayed.
         Kernel arguments are fixed by the graph: rows beyond the batch are padding (position
@@ -440,31 +471,41 @@ class StepRunner:
         self.rt.record(self.meta_copied)
         if tokens_from is not None:
             self.rt.copy_d2d(self.meta_dev.ptr + off["tokens"] * 4, tokens_from, R * 4)
-        if self.graph_logits is None:
+        picks = self._pick_buffers(bucket) if pick else None
+        if self.graph_logits is None and picks is None:
             self.graph_logits = self.rt.empty((self.max_seqs, self.vocab), F32)
-        out = self.graph_logits.rows(0, bucket)
-        graph = self.graphs.get((bucket, covered))
+        out = self.graph_logits.rows(0, bucket) if picks is None else None
+
+        def result():
+            if picks is not None:
+                return self.pick_ids.rows(0, n_rows)
+            return self._argmax_of(self.graph_logits.rows(0, n_rows), n_rows) if pick else self.graph_logits.rows(0, n_rows)
+        # a graph that picks holds other launches than one that writes logits: a key of its own
+        mode = "pick" if picks is not None else "logits"
+        graph = self.graphs.get((bucket, covered) if mode == "logits" else (bucket, covered, mode))
         if graph is not None:
             self.rt.graph_launch(graph)
-            return self.graph_logits.rows(0, n_rows)
+            self.graph_runs += 1
+            return result()
         ctx = self._context(off, bucket, bucket, host_entries, 1, covered, 0)
         self.arena.reset()
-        if bucket not in self.graphs:           # first time: eager, lets the arena grow
-            self.model.forward(ctx, self.caches, ctx.logit_rows, bucket, out)
-            self.graphs[bucket] = "warm"
-            return self.graph_logits.rows(0, n_rows)
+        warm = bucket if mode == "logits" else (bucket, mode)
+        if warm not in self.graphs:             # first time: eager, lets the arena grow
+            self.model.forward(ctx, self.caches, ctx.logit_rows, bucket, out, pick=picks)
+            self.graphs[warm] = "warm"
+            return result()
         self.arena.frozen = True
         try:
             self.rt.capture_begin()
             try:
-                self.model.forward(ctx, self.caches, ctx.logit_rows, bucket, out)
+                self.model.forward(ctx, self.caches, ctx.logit_rows, bucket, out, pick=picks)
             finally:
                 graph = self.rt.capture_end()
         finally:
             self.arena.frozen = False
-        self.graphs[(bucket, covered)] = graph
+        self.graphs[(bucket, covered) if mode == "logits" else (bucket, covered, mode)] = graph
         self.rt.graph_launch(graph)
-        return self.graph_logits.rows(0, n_rows)
+        return result()
 
     def close(self) -> None:
         """Gives back what lives outside the runtime's memory pools: the captured graphs and
@@ -479,23 +520,38 @@ class StepRunner:
         self.steplists.clear()
 
     MAX_STEPLISTS = 256
+    MAX_SIGHTED = 4096
 
-    def _forward(self, ctx, n_rows: int, out: Tensor, shape: tuple) -> None:
+    def _forward(self, ctx, n_rows: int, out: Optional[Tensor], shape: tuple, pick=None) -> None:
         """The model on an eager step.  Device addresses follow from the step's shape (the
         arena hands out the same addresses for the same sequence of sizes, the step's arrays
         lie at offsets fixed by the numbers of tokens and requests), so a shape that was seen
-        before is launched from its written-down list."""
+        before is launched from its written-down list.  A step of single tokens is written down
+        at once (its shape comes back as long as the same requests decode); any other shape
+        when it comes a second time (a mixed step's shape often never comes back, and writing
+        costs as much again as the launches).  Of 256 lists the one not used for the longest
+        time makes room for a new one, so the shapes that keep coming stay."""
         if not self.use_steplists:
-            self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, out)
+            self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, out, pick=pick)
+            self.steplist_misses += 1
             return
-        handle = self.steplists.get(shape)
+        handle = self.steplists.pop(shape, None)
         if handle is not None:
+            self.steplists[shape] = handle           # the most recently used one is the last
             self.k.steplist_run(handle, ctx.stream)
             self.steplist_runs += 1
             return
+        self.steplist_misses += 1
+        if shape[0] != shape[1] and shape not in self._sighted:          # more tokens than requests: not a decode step
+            if len(self._sighted) >= self.MAX_SIGHTED:
+                self._sighted.pop(next(iter(self._sighted)))
+            self._sighted[shape] = None
+            self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, out, pick=pick)
+            return
+        self._sighted.pop(shape, None)
         self.k.steplist_begin()
         try:
-            self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, out)
+            self.model.forward(ctx, self.caches, ctx.logit_rows, n_rows, out, pick=pick)
         except BaseException:
             h = self.k.steplist_end()
             if h is not None:
@@ -515,15 +571,22 @@ class StepRunner:
             self.k.steplist_destroy(self.steplists.pop(old))
         self.steplists[shape] = handle
 
-    def step(self, entries: Sequence[StepEntry], download: bool = True, tokens_from: Optional[int] = None):
+    def step(self, entries: Sequence[StepEntry], download: bool = True, tokens_from: Optional[int] = None,
+             pick: bool = False):
         """Run one step.  Returns float32 logits [wanted, vocab] on the host
         (``download=False``: the device tensor, valid until the next step).
+        ``pick``: the step wants nothing but the greedy choice of every wanted row; what comes
+        back is int32 ids [wanted] instead (the lowest index among a row's largest logits).
+        Where the model's head can, the ids are taken in the head product's epilogue and the
+        logits never reach memory; elsewhere they are written and an argmax kernel reads them.
         ``tokens_from``: a device pointer to int32 token ids, one per entry in the order of the
         entries, for a step in which every entry brings one token: the ids the last step's
         sampling kernel left on the device are fed without a trip to the host (the entries'
         own token values are then placeholders)."""
         entries = [e for e in entries if len(e.tokens) > 0]
         if not entries:
+            if pick:
+                return np.zeros((0,), np.int32) if download else None
             return np.zeros((0, self.vocab), np.float32) if download else None
         m = self.manager
         seen = set()
@@ -554,18 +617,26 @@ class StepRunner:
         self.rt.wait_event(self.meta_copied)     # the last step's copy has left the host buffer
         bucket = self._graph_bucket(entries)
         if bucket:
-            out = self._graph_step(entries, bucket, tokens_from)
+            out = self._graph_step(entries, bucket, tokens_from, pick)
         else:
             off, words, T, R, n_rows, host_entries, max_q, max_ctx, n_multi = self._pack(entries, T, R)
-            self._ensure_logits(n_rows)
+            picks = self._pick_buffers(n_rows) if pick and n_rows else None
+            if picks is None:
+                self._ensure_logits(n_rows)
             self.rt.copy_h2d_async(self.meta_dev.ptr, self.meta_host.ptr, words * 4)
             self.rt.record(self.meta_copied)
             if tokens_from is not None:
                 self.rt.copy_d2d(self.meta_dev.ptr + off["tokens"] * 4, tokens_from, R * 4)
             ctx = self._context(off, T, R, host_entries, max_q, max_ctx, n_multi)
             self.arena.reset()
-            out = self.logits.rows(0, n_rows)
-            self._forward(ctx, n_rows, out, (T, R, n_rows, n_multi, max_q, max_ctx, out.ptr))
+            if picks is not None:
+                self._forward(ctx, n_rows, None, (T, R, n_rows, n_multi, max_q, max_ctx, "pick", picks[0].ptr), pick=picks)
+                out = self.pick_ids.rows(0, n_rows)
+            else:
+                out = self.logits.rows(0, n_rows)
+                self._forward(ctx, n_rows, out, (T, R, n_rows, n_multi, max_q, max_ctx, out.ptr))
+                if pick:
+                    out = self._argmax_of(out, n_rows)
         for e in entries:
             m.commit(e.req, m.computed(e.req) + len(e.tokens))
         self.steps_run += 1

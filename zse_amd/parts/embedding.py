@@ -68,6 +68,28 @@ class LMHead(Part):
         self.weight = (weights.matrix([self.spec.weight], strip=True) if strip and strip(self.spec.hidden_size)
                        else weights.matrix([self.spec.weight]))
 
+    PICK_ROWS = 64         # the most rows the picking product takes
+
+    def can_pick(self, ctx, rows: int) -> bool:
+        """Whether ``pick`` serves this many rows: the matrix-core product with the picking
+        epilogue (up to 64 rows; more than 16 need the strip layout)."""
+        return bool(tuned_gemm(ctx, self.spec.hidden_size) and ctx.k.has("zk_head_pick_bf16") and
+                    1 <= rows <= self.PICK_ROWS and (rows <= 16 or self.weight.layout == "strip"))
+
+    def pick_scratch_bytes(self, kernels, rows: int) -> int:
+        return int(kernels.zk_head_pick_bf16_workspace(int(rows), self.spec.vocab_size))
+
+    def pick(self, ctx, x: Tensor, ids: Tensor, scratch: Tensor) -> Tensor:
+        """ids[r] = the column of row r's largest logit (after the soft cap; the lowest column
+        among equals): the greedy choice, taken in the product's epilogue strip by strip, so
+        that the [rows, vocab] logits are neither written nor read back.  The same column as
+        ``forward`` followed by the argmax kernel gives."""
+        s = self.spec
+        ctx.k.zk_head_pick_bf16(x.ptr, s.hidden_size, self.weight.ptr, x.shape[0], s.vocab_size, s.hidden_size,
+                                float(s.softcap) if s.softcap else 0.0, 1 if self.weight.layout == "strip" else 0,
+                                scratch.ptr, scratch.nbytes, ids.ptr, ctx.stream)
+        return ids
+
     def forward(self, ctx, x: Tensor, out: Tensor) -> Tensor:
         """x: normed rows [K, hidden]; out: float logits [K, vocab]."""
         s = self.spec

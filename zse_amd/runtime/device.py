@@ -166,6 +166,7 @@ BF16_KERNEL_SIGNATURES = {
     "zk_gemm_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, C.c_size_t, C.POINTER(C.c_int), _VP],
     "zk_gemm_bf16_static": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP],
     "zk_strip_layout": [_VP, _VP, _I, _I, _VP],
+    "zk_head_pick_bf16": [_VP, _I, _VP, _I, _I, _I, _F, _I, _VP, _SZ, _VP, _VP],
     "zk_probe_mfma_bf16": [_I, _VP, C.POINTER(C.c_double), _VP],
     "zk_qkv_rope_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "zk_attention_bf16": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
@@ -261,6 +262,9 @@ class KernelLibrary:
             self._dll.zk_qkv_rope_bf16_supports.restype = C.c_int
             self._dll.zk_qkv_rope_bf16_supports.argtypes = [_I, _I, _I, _I]
             self.zk_qkv_rope_bf16_supports = self._dll.zk_qkv_rope_bf16_supports
+            self._dll.zk_head_pick_bf16_workspace.restype = C.c_size_t
+            self._dll.zk_head_pick_bf16_workspace.argtypes = [_I, _I]
+            self.zk_head_pick_bf16_workspace = self._dll.zk_head_pick_bf16_workspace
             self._dll.zk_gemm_bf16_workspace.restype = C.c_size_t
             self._dll.zk_gemm_bf16_workspace.argtypes = []
             self.zk_gemm_bf16_workspace = self._dll.zk_gemm_bf16_workspace

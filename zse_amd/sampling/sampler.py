@@ -165,6 +165,11 @@ class DeviceSampler:
     # ---- a run of steps without waiting for the host in between
     RING = 16       # results that may be on their way to the host at a time
 
+    @property
+    def run_is_greedy(self) -> bool:
+        """Whether the run that ``prepare_run`` prepared takes the largest logit of every row."""
+        return bool(getattr(self, "_run_greedy", False))
+
     def can_defer(self, rows: Sequence[dict]) -> bool:
         """True when ``sample_deferred`` serves these rows: no penalties, and all greedy or all
         drawn."""
@@ -192,6 +197,22 @@ class DeviceSampler:
             self._run_u = self.rt.empty((max(flat.size, self.max_rows * 8),), F64)
         self.rt.copy_h2d(self._run_u.ptr, flat)
 
+    def ids_deferred(self, ids) -> "PendingIds":
+        """Ids that a step picked itself (``StepRunner.step(pick=True)``, device int32 [n]) on
+        their way to the host: as ``sample_deferred`` of a greedy run, without its kernels."""
+        return self._send(ids, ids.shape[0])
+
+    def _send(self, dev, n: int) -> "PendingIds":
+        rt = self.rt
+        if getattr(self, "_ring", None) is None:
+            self._ring = [(rt.pinned(self.max_rows * 4), rt.event()) for _ in range(self.RING)]
+            self._ring_at = 0
+        host, ev = self._ring[self._ring_at % self.RING]
+        self._ring_at += 1
+        rt.copy_d2h_async(host.ptr, dev.ptr, n * 4)
+        rt.record(ev)
+        return PendingIds(rt, dev.ptr, host, ev, n)
+
     def sample_deferred(self, logits, step_in_run: int) -> "PendingIds":
         """Enqueue the sampling of one step of a prepared run.  The ids stay on the device
         (``.device_ptr``, valid until the next call) and travel to the host behind the
@@ -208,14 +229,7 @@ class DeviceSampler:
                         self.keep_from.ptr if self._run_cut else None, self.keep_ties.ptr if self._run_cut else None,
                         self.ids2.ptr, n, V, self.scratch.ptr, rt.stream)
             dev = self.ids2
-        if getattr(self, "_ring", None) is None:
-            self._ring = [(rt.pinned(self.max_rows * 4), rt.event()) for _ in range(self.RING)]
-            self._ring_at = 0
-        host, ev = self._ring[self._ring_at % self.RING]
-        self._ring_at += 1
-        rt.copy_d2h_async(host.ptr, dev.ptr, n * 4)
-        rt.record(ev)
-        return PendingIds(rt, dev.ptr, host, ev, n)
+        return self._send(dev, n)
 
     def sample(self, logits, rows: Sequence[dict]) -> List[int]:
         """``logits``: device float32 [n, vocab]; ``rows``: per row a dict with
