@@ -461,6 +461,42 @@ def test_steps_launched_from_their_written_down_lists(cases, dtype):
         assert_close(listed_rows[r], refs[r][:n], dtype, f"listed {r}")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_a_step_that_picks_gives_the_argmax_of_its_logits(cases, name, dtype):
+    """``step(pick=True)`` against ``step()`` followed by NumPy's argmax (which keeps the first of
+    equal values too): prompt portions that want several rows, single tokens through graphs and
+    through launch lists, more wanted rows than the runner has places.  In bfloat16 the ids come
+    from the head product's epilogue and the logits are never written; in 32-bit an argmax kernel
+    reads them."""
+    from zse_amd.engine.runner import StepEntry
+    folder, streams, refs = cases[(name, dtype)]
+    reqs = ["r0", "r1", "r2", "r3", "r4"]
+
+    def run(pick):
+        runner = make_runner(folder, dtype, page_size=PAGE[name], cache_tokens=1024, max_seqs=5,
+                             max_batch_tokens=256, max_model_len=256, use_graphs=True)
+        out = []
+        # every row of five prompts' first 12 tokens: 60 wanted rows, five places
+        out.append(runner.step([StepEntry(r, streams[r][:12], range(12)) for r in reqs], pick=pick))
+        fed = {r: 12 for r in reqs}
+        for i in range(9):
+            live = reqs if i % 4 != 3 else reqs[:3]
+            out.append(runner.step([StepEntry(r, [streams[r][fed[r]]], [0]) for r in live], pick=pick))
+            for r in live:
+                fed[r] += 1
+        if pick and dtype == "bfloat16":
+            assert any(len(k) == 3 and k[2] == "pick" for k, g in runner.graphs.items() if isinstance(g, int))
+            assert runner.graph_logits is None and runner.pick_scratch is not None
+        runner.close()
+        return out
+
+    logits, ids = run(False), run(True)
+    for z, got in zip(logits, ids):
+        assert got.dtype == np.int32 and got.shape == (z.shape[0],)
+        assert np.array_equal(got, z.argmax(axis=1))
+
+
 def test_a_tensor_dropped_during_capture_is_freed_after_it():
     """Freeing device memory synchronizes, which a capturing stream does not allow; the garbage
     collector may drop a tensor at any moment, also in the middle of a capture.  Such frees wait

@@ -416,10 +416,13 @@ class StepRunner:
         """(ids, scratch) if the model's head picks for ``rows`` rows without writing logits,
         else None (the step then writes logits and the argmax kernel reads them)."""
         head = self.model.head
-        if self.pick_ids is None:
-            self.pick_ids = self.rt.empty((max(self.max_seqs, 8),), I32)
-            self.argmax_scratch = self.rt.empty((max(self.max_seqs, 8) * 64 * 2,), F32)
-        if not hasattr(head, "can_pick") or rows > self.pick_ids.shape[0]:
+        if self.pick_ids is None or self.pick_ids.shape[0] < rows:
+            # room for the ids of every wanted row (a step may want more rows than it has requests)
+            self.rt.sync()
+            room = max(rows, self.max_seqs, 8)
+            self.pick_ids = self.rt.empty((room,), I32)
+            self.argmax_scratch = self.rt.empty((room * 64 * 2,), F32)
+        if not hasattr(head, "can_pick"):
             return None
         if rows not in self._head_picks:
             self._head_picks[rows] = bool(head.can_pick(StepContext(self), rows))
