@@ -281,11 +281,11 @@ def run_workload(name, a, model=None):
 class Timed:
     """A model on a runner sized for the batches and the context that are timed."""
 
-    def __init__(self, model, rt, cfg, max_b, context, prefill_tokens, graphs):
+    def __init__(self, model, rt, cfg, max_b, context, prefill_tokens, graphs, page=16):
         from zse_amd.engine.runner import StepRunner
         from zse_amd.sampling.sampler import DeviceSampler
         self.model, self.rt, self.cfg, self.context, self.T = model, rt, cfg, context, prefill_tokens
-        self.V, page = cfg["vocab_size"], 16
+        self.V = cfg["vocab_size"]
         longest = max(context, prefill_tokens)       # a prompt longer than the decode context still fits
         self.runner = StepRunner(model, rt, "bfloat16", page_size=page,
                                  num_pages=max(max_b * (-(-context // page) + 1), -(-longest // page)) + 8,
@@ -433,6 +433,7 @@ def main():
     ap.add_argument("--no-check", action="store_true", help="profiling aid: skip the check before timing")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="profiling aid: run one of the two workloads (the JSON line then lacks the other)")
+    ap.add_argument("--page-size", type=int, default=16, help="tokens a page of the cache holds")
     ap.add_argument("--quick", action="store_true",
                     help="the headline alone: no decode at context 8,192, no 9B and 27B figures")
     a = ap.parse_args()
@@ -474,7 +475,7 @@ def main():
     log(f"probes: {peak_bw / 1e9:.0f} GB/s streamed, {peak_fl / 1e12:.0f} TFLOP/s bf16 on the matrix cores")
 
     max_b = max(points)
-    t = Timed(model, rt, cfg, max_b, a.context, a.prefill_tokens, not a.no_graphs)
+    t = Timed(model, rt, cfg, max_b, a.context, a.prefill_tokens, not a.no_graphs, page=a.page_size)
     runner = t.runner
     log(f"model ready in {time.time() - t0:.1f} s: {cfg['num_hidden_layers']} layers, "
         f"{model.weight_bytes / 1e9:.2f} GB of weights, cache {runner.cache_bytes() / 1e9:.2f} GB")
@@ -514,7 +515,7 @@ def main():
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": dict(shape_of(cfg, full_layers), model=f"gemma2-{a.model}-shapes-random", global_batch=a.batch,
-                       seq_len=a.context, prompt_len=a.prefill_tokens, page_size=16, parallelism="single-gpu",
+                       seq_len=a.context, prompt_len=a.prefill_tokens, page_size=a.page_size, parallelism="single-gpu",
                        graphs=int(not a.no_graphs), graph_max_batch=graph_max_batch),
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(byts / step_s / 1e9, 1), "peak": PEAK_HBM / 1e9,
