@@ -1102,3 +1102,67 @@ def test_a_model_made_on_the_device_equals_the_folder_written_on_the_host(rt, tm
                                 max_model_len=64, use_graphs=False)
             rows.append(runner.step([StepEntry("a", toks, range(len(toks)))]))
         assert np.abs(rows[0]).max() > 0.1 and np.array_equal(rows[0], rows[1]), dtype
+
+
+def test_the_two_ways_to_the_cut_offs(rt):
+    """Rows made for the borders between the short way (a few candidates near the maximum, sorted by
+    one block) and the long way (the search over the whole row): as many equal logits at the top as
+    the candidates' room holds and one more, a k-th largest logit far below the maximum, a row of a
+    real model's kind (a few hundred likely tokens over a flat rest), logits on the edges of the
+    histogram's buckets, NaN among them.  Each row goes the way it is meant to and draws what the
+    host implementation draws."""
+    from zse_amd.sampling import DeviceSampler, SamplingParams, sample_host, uniform
+    rng = np.random.default_rng(21)
+    V = 70001
+    cap = 2048
+    def base():
+        return (rng.normal(size=V) * 2 - 40).astype(np.float32)
+    cases = []            # (logits, params, the way)
+    full = base(); full[rng.choice(V, cap, replace=False)] = 3.0
+    cases.append((full, dict(top_k=cap, top_p=0.7), 1))
+    cases.append((full, dict(top_k=100), 1))
+    over = base(); over[rng.choice(V, cap + 1, replace=False)] = 3.0
+    cases.append((over, dict(top_k=100, top_p=0.9), 2))
+    far = (rng.normal(size=V) * 2).astype(np.float32); far[12345] = 90.0
+    cases.append((far, dict(top_k=50), 2))
+    cases.append((far, dict(top_p=0.9), 1))                   # one logit holds it all
+    peaked = base(); idx = rng.choice(V, 300, replace=False); peaked[idx] = (rng.normal(size=300) * 3).astype(np.float32)
+    cases.append((peaked, dict(top_p=0.9), 1))
+    cases.append((peaked, dict(top_k=50, top_p=0.9), 1))
+    cases.append((peaked, dict(top_k=50), 1))
+    cases.append((peaked, dict(top_p=0.999999), 1))             # what lies 32 below the maximum weighs nothing
+    edges = base(); edges[:1500] = (5.0 - np.arange(1500) / 32.0 * 0.8).astype(np.float32)      # temperature 0.8: steps of a bucket
+    cases.append((edges, dict(top_k=700), 1))
+    cases.append((edges, dict(top_p=0.95), 1))
+    cases.append((edges, dict(top_k=1000, top_p=0.99), 1))
+    cases.append((edges, dict(top_k=1500, top_p=0.99), 2))    # the k-th largest lies in the last bucket
+    nans = peaked.copy(); nans[rng.choice(V, 50, replace=False)] = np.nan; nans[idx[:3]] = np.nan
+    cases.append((nans, dict(top_k=20, top_p=0.8), 1))
+    spread = (rng.normal(size=V) * 0.5).astype(np.float32)      # many logits above either cut-off, few in its bucket
+    cases.append((spread, dict(top_p=0.9), 3))
+    cases.append((spread, dict(top_k=5000), 3))
+    cases.append((spread, dict(top_k=5000, top_p=0.9), 2))
+    grid = (np.round(spread * 80) / 80).astype(np.float32)      # some hundred equal logits at the cut-off
+    cases.append((grid, dict(top_p=0.8), 3))
+    cases.append((grid, dict(top_k=3000), 3))
+    flat = np.zeros(V, np.float32)
+    cases.append((flat, dict(top_k=10), 2))
+    cases.append((flat, dict(top_p=0.5005), 2))
+    cases.append((flat, dict(), 0))
+    z = np.stack([c[0] for c in cases])
+    params = [SamplingParams(temperature=0.8, **c[1]) for c in cases]
+    sampler = DeviceSampler(rt, rt.kernels("float32"), len(cases) + 3)
+    for trial in range(6):
+        us = [(0.0, 0.999999)[trial] if trial < 2 else uniform(trial, i) for i in range(len(cases))]
+        rows = [{"params": p_, "u": u_, "past": ()} for p_, u_ in zip(params, us)]
+        got = sampler.sample(rt.upload(z), rows)
+        assert sampler.cut_ways(len(cases)) == [c[2] for c in cases]
+        zz = np.where(np.isnan(z), -np.inf, z)                 # the host implementation has no rule for NaN: never drawn
+        want = [sample_host(zz[i], r["params"], r["u"]) for i, r in enumerate(rows)]
+        assert got == want, [(i, cases[i][1], g, w) for i, (g, w) in enumerate(zip(got, want)) if g != w]
+    # fewer rows afterwards, and more again: what a call leaves behind serves the next
+    for n in (2, len(cases)):
+        rows = [{"params": params[i], "u": uniform(99, i), "past": ()} for i in range(n)]
+        got = sampler.sample(rt.upload(z[:n]), rows)
+        zz = np.where(np.isnan(z), -np.inf, z)
+        assert got == [sample_host(zz[i], r["params"], r["u"]) for i, r in enumerate(rows)]

@@ -202,7 +202,7 @@ class Engine:
         reqs = [s.request for s in plan.items]
         first_len = [len(r.output_tokens) for r in reqs]
         sampler.prepare_run(self._rows(plan), [[uniform(r.seed, n0 + i) for r, n0 in zip(reqs, first_len)]
-                                               for i in range(length)])
+                                               for i in range(length)], vocab=runner.vocab)
         pending, done, tokens_from = [], [], None
         for i in range(length):
             known = tokens_from is None

@@ -157,7 +157,7 @@ KERNEL_SIGNATURES = {
                            _I, _I, _VP],
     "zk_argmax": [_VP, _VP, _I, _I, _VP, _VP],
     "zk_sample": [_VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP],
-    "zk_sample_cutoff": [_VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP],
+    "zk_sample_cut": [_VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _I, _VP],
     "zk_penalize": [_VP, _I, _VP, _VP, _VP, _I, _VP],
     "zk_probe_read": [_VP, _SZ, _VP, _VP],
 }
@@ -239,9 +239,13 @@ class KernelLibrary:
             fn.argtypes = args
             fn.restype = C.c_int
             setattr(self, name, self._wrap(name, fn))
-        for name in ("zk_sample_scratch_bytes", "zk_sample_cutoff_scratch_bytes"):
+        for name in ("zk_sample_scratch_bytes", "zk_sample_cut_scratch_bytes"):
             fn = getattr(self._dll, name)
             fn.restype, fn.argtypes = C.c_size_t, [_I]
+            setattr(self, name, fn)
+        for name in ("zk_sample_cut_row_bytes", "zk_sample_cut_mode_offset"):
+            fn = getattr(self._dll, name)
+            fn.restype, fn.argtypes = C.c_size_t, []
             setattr(self, name, fn)
         if dtype == BF16:
             self._dll.zk_attention_bf16_supports.restype = C.c_int

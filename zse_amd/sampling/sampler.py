@@ -12,8 +12,9 @@ output token) instead of coming from one shared generator (:30-31), so a
 request samples the same tokens whatever else is in the batch.
 
 All of it runs on the device (csrc/sampling.hip): the penalty as a small
-kernel over the (row, token) pairs, top-k and top-p as a cut-off value and a
-number of its ties per row, then the argmax or the inverse CDF.  The host
+kernel over the (row, token) pairs, then the argmax, the inverse CDF, or, for
+rows with top-k or top-p, the kernels that find both cut-offs and draw among
+what they leave.  The host
 implementation below is the same arithmetic in float64 and what the device is
 tested against; the reference samples everything on the host (:10-11).
 """
@@ -147,11 +148,9 @@ class DeviceSampler:
         self.temp = rt.empty((max_rows,), F32)
         self.u = rt.empty((max_rows,), F64)
         self.scratch = rt.empty(((kernels.zk_sample_scratch_bytes(max_rows) + 3) // 4,), F32)
-        self.cut_scratch = None                             # histograms of the cut-off search, on first use
+        self.cut_scratch = None                             # histograms and candidates of the cut-offs, on first use
         self.top_k = rt.empty((max_rows,), I32)
         self.top_p = rt.empty((max_rows,), F32)
-        self.keep_from = rt.empty((max_rows,), F32)
-        self.keep_ties = rt.empty((max_rows,), I32)
         self._pen = None                                    # (rows, tokens, scales) on the device, grown on demand
         # the rows' temperatures, uniform numbers and cut-offs on their way to the device: page-locked,
         # so their copies queue behind the step's kernels instead of waiting for them (``sample``
@@ -178,7 +177,18 @@ class DeviceSampler:
         kinds = {bool(r["params"].greedy) for r in rows}
         return len(kinds) == 1
 
-    def prepare_run(self, rows: Sequence[dict], us: Sequence[Sequence[float]]):
+    # Which kernels a batch needs.  The kernels themselves decide row by row (a top_k of the
+    # vocabulary's size or more is no top-k); the host only has to launch the one that serves a
+    # row, and without the vocabulary's size it launches both for a row with a top_k alone.
+    @staticmethod
+    def _has_cut(p: SamplingParams, vocab: Optional[int]) -> bool:
+        return p.top_p < 1.0 or (p.top_k > 0 and (vocab is None or p.top_k < vocab))
+
+    @staticmethod
+    def _is_plain(p: SamplingParams, vocab: Optional[int]) -> bool:
+        return p.top_p >= 1.0 and (p.top_k == 0 or vocab is None or p.top_k >= vocab)
+
+    def prepare_run(self, rows: Sequence[dict], us: Sequence[Sequence[float]], vocab: Optional[int] = None):
         """For a run of steps over the same rows: temperatures once, and the uniform numbers
         of every step of the run (``us[step][row]``), so that no step of the run copies
         anything from the host."""
@@ -188,7 +198,8 @@ class DeviceSampler:
         if self._run_greedy:
             return
         self.rt.copy_h2d(self.temp.ptr, np.array([r["params"].temperature for r in rows], dtype=np.float32))
-        self._run_cut = any(r["params"].top_k > 0 or r["params"].top_p < 1.0 for r in rows)
+        self._run_cut = any(self._has_cut(r["params"], None) for r in rows)
+        self._run_plain = any(self._is_plain(r["params"], vocab) for r in rows)
         if self._run_cut:
             self.rt.copy_h2d(self.top_k.ptr, np.array([r["params"].top_k for r in rows], dtype=np.int32))
             self.rt.copy_h2d(self.top_p.ptr, np.array([r["params"].top_p for r in rows], dtype=np.float32))
@@ -223,11 +234,7 @@ class DeviceSampler:
             k.zk_argmax(logits.ptr, self.ids.ptr, n, V, self.scratch.ptr, rt.stream)
             dev = self.ids
         else:
-            if self._run_cut:
-                self._cutoff(logits, n, V)
-            k.zk_sample(logits.ptr, self.temp.ptr, self._run_u.ptr + step_in_run * n * 8,
-                        self.keep_from.ptr if self._run_cut else None, self.keep_ties.ptr if self._run_cut else None,
-                        self.ids2.ptr, n, V, self.scratch.ptr, rt.stream)
+            self._draw(logits, n, V, self._run_u.ptr + step_in_run * n * 8, self._run_cut, self._run_plain)
             dev = self.ids2
         return self._send(dev, n)
 
@@ -254,26 +261,42 @@ class DeviceSampler:
             self._stage_u[:n] = [r["u"] for r in rows]
             rt.copy_h2d_async(self.temp.ptr, st + self.max_rows * 8, n * 4)
             rt.copy_h2d_async(self.u.ptr, st, n * 8)
-            cut = any(not g and (r["params"].top_k > 0 or r["params"].top_p < 1.0) for r, g in zip(rows, greedy))
+            cut = any(not g and self._has_cut(r["params"], V) for r, g in zip(rows, greedy))
+            plain = any(not g and self._is_plain(r["params"], V) for r, g in zip(rows, greedy))
             if cut:
-                self._stage_k[:n] = [0 if g else r["params"].top_k for r, g in zip(rows, greedy)]
+                # (a greedy row, whose draw nobody reads, as top-k 1: the cheapest there is)
+                self._stage_k[:n] = [1 if g else r["params"].top_k for r, g in zip(rows, greedy)]
                 self._stage_p[:n] = [1.0 if g else r["params"].top_p for r, g in zip(rows, greedy)]
                 rt.copy_h2d_async(self.top_k.ptr, st + self.max_rows * 12, n * 4)
                 rt.copy_h2d_async(self.top_p.ptr, st + self.max_rows * 16, n * 4)
-                self._cutoff(logits, n, V)
-            k.zk_sample(logits.ptr, self.temp.ptr, self.u.ptr, self.keep_from.ptr if cut else None,
-                        self.keep_ties.ptr if cut else None, self.ids2.ptr, n, V, self.scratch.ptr, rt.stream)
+            self._draw(logits, n, V, self.u.ptr, cut, plain)
         g = rt.download(self.ids.rows(0, n)) if any(greedy) else None
         s = rt.download(self.ids2.rows(0, n)) if not all(greedy) else None
         return [int(g[i]) if greedy[i] else int(s[i]) for i in range(n)]
 
-    def _cutoff(self, logits, n: int, V: int) -> None:
-        """top-k / top-p of the rows (``self.top_k``, ``self.top_p``) as ``keep_from`` / ``keep_ties``."""
-        from ..runtime.device import F32
-        if self.cut_scratch is None:
-            self.cut_scratch = self.rt.empty(((self.k.zk_sample_cutoff_scratch_bytes(self.max_rows) + 3) // 4,), F32)
-        self.k.zk_sample_cutoff(logits.ptr, self.temp.ptr, self.top_k.ptr, self.top_p.ptr, self.keep_from.ptr,
-                                self.keep_ties.ptr, n, V, self.cut_scratch.ptr, self.rt.stream)
+    def _draw(self, logits, n: int, V: int, u_ptr: int, cut: bool, plain: bool) -> None:
+        """Ids of the rows into ``self.ids2``.  ``cut``: some rows have top-k or top-p
+        (``self.top_k``, ``self.top_p``); ``plain``: some have neither."""
+        k, rt = self.k, self.rt
+        if plain or not cut:
+            k.zk_sample(logits.ptr, self.temp.ptr, u_ptr, self.top_k.ptr if cut else None, self.top_p.ptr if cut else None,
+                        self.ids2.ptr, n, V, self.scratch.ptr, rt.stream)
+        if not cut:
+            return
+        if self.cut_scratch is None:        # zero at first, and left so by every call
+            from ..runtime.device import F32
+            self.cut_scratch = rt.zeros(((k.zk_sample_cut_scratch_bytes(self.max_rows) + 3) // 4,), F32)
+        k.zk_sample_cut(logits.ptr, self.temp.ptr, u_ptr, self.top_k.ptr, self.top_p.ptr, self.ids2.ptr, n, V,
+                        self.cut_scratch.ptr, self.max_rows, rt.stream)
+
+    def cut_ways(self, n: int) -> List[int]:
+        """Which way each of the last ``n`` rows drawn with cut-offs went (0: it had none, 1: the
+        candidates, 2: the search over the whole row); for tests and measurements."""
+        k = self.k
+        words = self.rt.download(self.cut_scratch).view(np.int32)
+        at = k.zk_sample_cut_mode_offset() // 4
+        row_words = k.zk_sample_cut_row_bytes() // 4
+        return [int(words[r * row_words + at]) for r in range(n)]
 
     def _penalize(self, logits, V: int, pen) -> None:
         from ..runtime.device import F32, I32
