@@ -39,6 +39,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 PEAK_HBM = 8.0e12          # bytes/s, MI355X
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+REFERENCE_SAMPLING = {"temperature": 1.0, "top_k": 50, "top_p": 0.9}     # the reference's defaults
 
 GEMMA2_2B = dict(
     architectures=["Gemma2ForCausalLM"], model_type="gemma2", num_hidden_layers=26, hidden_size=2304,
@@ -326,9 +327,11 @@ class Timed:
                     for at in range(0, T, portion))
         return float(np.median(times[1:])), flops
 
-    def decode(self, B, steps, warmup):
+    def decode(self, B, steps, warmup, drawn=None):
         """``steps`` decode steps of ``B`` requests that end at the full context: (tokens a
-        second, seconds a step, bytes a step has to read, how the steps were launched)."""
+        second, seconds a step, bytes a step has to read, how the steps were launched).
+        ``drawn``: keyword arguments of SamplingParams for steps that draw their tokens instead of
+        taking the largest logit."""
         from zse_amd.engine.runner import StepEntry
         from zse_amd.sampling.sampler import SamplingParams
         runner, rt, sampler, rng, V = self.runner, self.rt, self.sampler, self.rng, self.V
@@ -341,19 +344,24 @@ class Timed:
                 runner.step([StepEntry(r, rng.integers(0, V, n).tolist(), [])], download=False)
                 left -= n
         first = rng.integers(0, V, B).tolist()
-        rows = [{"params": SamplingParams(temperature=0.0), "u": 0.0} for _ in range(B)]
-        # As the engine decodes greedily: the step picks the largest logits itself and leaves the
-        # ids on the device, the next step takes them from there, and the host reads them four
-        # steps at a time (it has to, for stop tokens) while the next steps are already enqueued.
-        sampler.prepare_run(rows, [[0.0] * B])
-        pending, fed = [], None
+        rows = [{"params": SamplingParams(**(drawn or {"temperature": 0.0})), "u": 0.0} for _ in range(B)]
+        # As the engine decodes: a greedy step picks the largest logits itself, a drawing step hands
+        # its logits to the sampling kernels; either way the ids stay on the device, the next step
+        # takes them from there, and the host reads them four steps at a time (it has to, for stop
+        # tokens) while the next steps are already enqueued.
+        us = rng.random((4, B)).tolist()
+        sampler.prepare_run(rows, us, vocab=V)
+        pending, fed, turn = [], None, 0
 
         def one():
-            nonlocal fed
+            nonlocal fed, turn
             toks = first if fed is None else [0] * B
-            picked = runner.step([StepEntry(r, [t], [0]) for r, t in zip(reqs, toks)], download=False,
-                                 tokens_from=fed, pick=True)
-            ids = sampler.ids_deferred(picked)
+            entries = [StepEntry(r, [t], [0]) for r, t in zip(reqs, toks)]
+            if drawn:
+                ids = sampler.sample_deferred(runner.step(entries, download=False, tokens_from=fed), turn % 4)
+                turn += 1
+            else:
+                ids = sampler.ids_deferred(runner.step(entries, download=False, tokens_from=fed, pick=True))
             fed = ids.device_ptr
             pending.append(ids)
             if len(pending) == 4:
@@ -505,6 +513,11 @@ def main():
         results[B] = t.decode(B, k, w)
         log(f"decode batch {B}: {results[B][0]:.1f} tok/s, {results[B][1] * 1e3:.3f} ms/step, "
             f"{results[B][2] / results[B][1] / 1e9:.0f} GB/s ({results[B][3]})")
+    # the same at the reference's default sampling parameters (orchestrator/engine.py:40-43)
+    drawn = None
+    if not a.only and a.batch in points:
+        drawn = t.decode(a.batch, max(16, a.steps // 2), max(4, a.warmup // 2), drawn=REFERENCE_SAMPLING)
+        log(f"decode batch {a.batch}, drawn with {REFERENCE_SAMPLING}: {drawn[0]:.1f} tok/s, {drawn[1] * 1e3:.3f} ms/step")
     graph_max_batch = runner.graph_max_batch
     t.close()
 
@@ -524,6 +537,8 @@ def main():
         "points": {f"decode_b{B}": round(results[B][0], 1) for B in points if B != a.batch},
         "points_roofline_frac": {f"decode_b{B}": round(results[B][2] / results[B][1] / PEAK_HBM, 4) for B in points},
         "points_launched": {f"decode_b{B}": results[B][3] for B in points},
+        "drawn": None if drawn is None else dict(REFERENCE_SAMPLING, value=round(drawn[0], 1), batch=a.batch,
+                                                   ms_per_step=round(drawn[1] * 1e3, 4)),
         "probed": {"hbm_gbs": round(peak_bw / 1e9, 1), "mfma_bf16_tflops": round(peak_fl / 1e12, 1)},
         "checked": check is not None, "check": check,
     }
