@@ -853,6 +853,46 @@ def test_qkv_product_that_rotates_and_stores(rt, M, K, nh, nkv, hd, bs, vt, stri
     assert not k.zk_qkv_rope_bf16_supports(M, K, hd, hd // 2)
 
 
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("T,nh,nkv,hd,bs,vt,rot", [(5, 3, 1, 48, 8, 1, 48), (40, 8, 4, 64, 16, 1, 64), (64, 2, 2, 256, 16, 1, 256),
+                                                 (100, 4, 2, 32, 8, 0, 32), (23, 2, 1, 64, 4, 0, 32), (72, 3, 3, 16, 8, 1, 16)])
+def test_rotation_that_adds_up_partial_sums_itself(rt, dtype, T, nh, nkv, hd, bs, vt, rot):
+    """The rows of [q | k | v] as three planes of float partial sums, added up by the kernel that
+    rotates and stores: the same bits, in q and in the cache, as from the rows added up in order and
+    rounded to the storage type beforehand.  Eight tokens in a row land in eight slots in a row of
+    one page (the transposed store of whole groups) and one token is stored nowhere."""
+    k = rt.kernels(dtype)
+    rng = np.random.default_rng(T * 10 + hd)
+    width = (nh + 2 * nkv) * hd
+    planes = (rng.normal(size=(3, T, width)) * np.array([1.0, 1e-2, 1e-4])[:, None, None]).astype(np.float32)
+    summed = (planes[0] + planes[1]) + planes[2]
+    rows = bf16(summed) if dtype == "bfloat16" else summed
+    pages = (T + bs - 1) // bs + 3
+    free = [x for x in range(pages * bs) if x // bs != 2]
+    slots = rng.permutation(free)[:T].astype(np.int32)
+    if T >= 16 and bs >= 8:
+        slots[8:16] = 2 * bs + np.arange(8)
+    slots[min(3, T - 1)] = -1
+    pos = rng.integers(0, 5000, T).astype(np.int32)
+    inv = (1.0 / 10000.0 ** (2.0 * np.arange(rot // 2) / rot)).astype(np.float32)
+    P, S, I = rt.upload(pos), rt.upload(slots), rt.upload(inv)
+    pattern = rng.normal(size=(pages, nkv, bs, hd)).astype(np.float32)
+    got = []
+    for sums in (0, 3):
+        Q = up(rt, rows if not sums else np.zeros_like(rows), dtype)
+        KC = up(rt, pattern, dtype)
+        VC = up(rt, pattern.reshape(pages, nkv, hd, bs) if vt else pattern, dtype)
+        if sums:
+            k.zk_rope_cache_write_sums(Q.ptr, ptr(rt.upload(planes)), 3, P.ptr, S.ptr, I.ptr, rot, KC.ptr, VC.ptr, T, nh, nkv,
+                                       hd, bs, vt, rt.stream)
+        else:
+            k.zk_rope_cache_write(Q.ptr, P.ptr, S.ptr, I.ptr, rot, KC.ptr, VC.ptr, T, nh, nkv, hd, bs, vt, rt.stream)
+        got.append((rt.download_f32(Q)[:, :nh * hd], rt.download_f32(KC), rt.download_f32(VC)))
+    for x, y in zip(*got):
+        assert np.array_equal(x, y)
+    assert not np.array_equal(got[0][1], bf16(pattern) if dtype == "bfloat16" else pattern)      # something was stored
+
+
 def test_convert_and_fill(rt):
     rng = np.random.default_rng(0)
     x = rng.normal(size=1003).astype(np.float32)

@@ -453,14 +453,46 @@ __global__ void softcap_kernel(float* __restrict__ z, size_t n, float cap) {
 // (slot < 0: nothing stored).  Cache layout per layer: K [page][kv head][bs][hd];
 // V the same, or transposed [page][kv head][hd][bs] when v_transposed is set.
 
-__global__ void rope_cache_write_kernel(act_t* __restrict__ qkv, const int* __restrict__ positions,
+// Where the rows come from: the matrix itself, or (sums > 0) that many planes of [T, width]
+// float partial sums of a product that split K, added in order and rounded to the activation
+// type, which is what the product's own joining kernel would have stored.  q then goes to qkv.
+struct QkvSource {
+  const act_t* rows;
+  const float* planes;
+  int sums;
+  size_t plane;
+  __device__ __forceinline__ float at(size_t i) const {
+    if (sums <= 0) return to_f32(rows[i]);
+    float x = planes[i];
+    for (int p = 1; p < sums; p++) x += planes[p * plane + i];
+    return to_f32(from_f32<act_t>(x));
+  }
+  __device__ __forceinline__ void at4(size_t i, float v[4]) const {
+    if (sums <= 0) {
+      load4<act_t>(rows + i, v);
+      return;
+    }
+    load4<float>(planes + i, v);
+    for (int p = 1; p < sums; p++) {
+      float w[4];
+      load4<float>(planes + p * plane + i, w);
+#pragma unroll
+      for (int e = 0; e < 4; e++) v[e] += w[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] = to_f32(from_f32<act_t>(v[e]));
+  }
+};
+
+__global__ void rope_cache_write_kernel(act_t* __restrict__ qkv, QkvSource from, const int* __restrict__ positions,
                                         const int* __restrict__ slot_map,
                                         const float* __restrict__ inv_freq, int rotary_dim,
                                         act_t* __restrict__ kcache, act_t* __restrict__ vcache,
                                         int nh, int nkv, int hd, int bs, int v_transposed) {
   const int t = blockIdx.x;
   const int head = blockIdx.y;  // [0,nh): q; [nh, nh+nkv): k; [nh+nkv, nh+2nkv): v
-  act_t* src = qkv + (size_t)t * (nh + 2 * nkv) * hd + (size_t)head * hd;
+  const size_t at = (size_t)t * (nh + 2 * nkv) * hd + (size_t)head * hd;
+  act_t* q_out = qkv + at;
   const float pos = (float)positions[t];
   const int half = rotary_dim / 2;
   const int slot = slot_map ? slot_map[t] : -1;
@@ -471,7 +503,7 @@ __global__ void rope_cache_write_kernel(act_t* __restrict__ qkv, const int* __re
     const size_t page = slot / bs, off = slot % bs;
     if (head >= nh + nkv && v_transposed) {
       act_t* vt = vcache + (page * nkv + kvh) * (size_t)hd * bs + off;
-      for (int i = threadIdx.x; i < hd; i += blockDim.x) vt[(size_t)i * bs] = src[i];
+      for (int i = threadIdx.x; i < hd; i += blockDim.x) vt[(size_t)i * bs] = from_f32<act_t>(from.at(at + i));
       return;
     }
     dst = base + ((page * nkv + kvh) * bs + off) * hd;
@@ -481,22 +513,26 @@ __global__ void rope_cache_write_kernel(act_t* __restrict__ qkv, const int* __re
       const float ang = pos * inv_freq[i];
       float sn, cs;
       sincosf(ang, &sn, &cs);
-      const float a = to_f32(src[i]), b = to_f32(src[i + half]);
+      const float a = from.at(at + i), b = from.at(at + i + half);
       float fa, fb;
       rotate_pair(a, b, sn, cs, fa, fb);
       const act_t ra = from_f32<act_t>(fa), rb = from_f32<act_t>(fb);
       if (head < nh) {
-        src[i] = ra;
-        src[i + half] = rb;
+        q_out[i] = ra;
+        q_out[i + half] = rb;
       } else if (dst) {
         dst[i] = ra;
         dst[i + half] = rb;
       }
     }
-    if (head >= nh && dst)
-      for (int i = rotary_dim + threadIdx.x; i < hd; i += blockDim.x) dst[i] = src[i];
+    if (head < nh) {
+      if (from.sums > 0)      // what is not rotated still has to reach qkv
+        for (int i = rotary_dim + threadIdx.x; i < hd; i += blockDim.x) q_out[i] = from_f32<act_t>(from.at(at + i));
+    } else if (dst) {
+      for (int i = rotary_dim + threadIdx.x; i < hd; i += blockDim.x) dst[i] = from_f32<act_t>(from.at(at + i));
+    }
   } else if (dst) {
-    for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[i] = src[i];
+    for (int i = threadIdx.x; i < hd; i += blockDim.x) dst[i] = from_f32<act_t>(from.at(at + i));
   }
 }
 
@@ -505,7 +541,7 @@ __global__ void rope_cache_write_kernel(act_t* __restrict__ qkv, const int* __re
 // all heads, four values a load.
 #define ROPE_MAX_HALF 256
 __global__ __launch_bounds__(256) void rope_cache_write_token_kernel(
-    act_t* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ slot_map,
+    act_t* __restrict__ qkv, QkvSource from, const int* __restrict__ positions, const int* __restrict__ slot_map,
     const float* __restrict__ inv_freq, act_t* __restrict__ kcache, act_t* __restrict__ vcache, int nh,
     int nkv, int hd, int bs, int v_transposed) {
   __shared__ float s_sin[ROPE_MAX_HALF], s_cos[ROPE_MAX_HALF];
@@ -515,23 +551,23 @@ __global__ __launch_bounds__(256) void rope_cache_write_token_kernel(
   const int slot = slot_map ? slot_map[t] : -1;
   for (int i = tid; i < half; i += 256) sincosf(pos * inv_freq[i], &s_sin[i], &s_cos[i]);
   __syncthreads();
-  act_t* row = qkv + (size_t)t * (nh + 2 * nkv) * hd;
+  const size_t width = (size_t)(nh + 2 * nkv) * hd, row_at = (size_t)t * width;
+  act_t* row = qkv + row_at;
   const size_t page = slot >= 0 ? slot / bs : 0, off = slot >= 0 ? slot % bs : 0;
   // q and k heads: pieces of four pairs (i, i + half)
   const int ppr = half / 4;
   for (int it = tid; it < (nh + nkv) * ppr; it += 256) {
     const int head = it / ppr, i = (it % ppr) * 4;
-    act_t* src = row + (size_t)head * hd;
     float a[4], b[4], ra[4], rb[4];
-    load4<act_t>(src + i, a);
-    load4<act_t>(src + i + half, b);
+    from.at4(row_at + (size_t)head * hd + i, a);
+    from.at4(row_at + (size_t)head * hd + i + half, b);
 #pragma unroll
     for (int e = 0; e < 4; e++) {
       rotate_pair(a[e], b[e], s_sin[i + e], s_cos[i + e], ra[e], rb[e]);
     }
     if (head < nh) {
-      store4(src + i, ra);
-      store4(src + i + half, rb);
+      store4(row + (size_t)head * hd + i, ra);
+      store4(row + (size_t)head * hd + i + half, rb);
     } else if (slot >= 0) {
       act_t* dst = kcache + ((page * nkv + (head - nh)) * bs + off) * hd;
       store4(dst + i, ra);
@@ -554,14 +590,14 @@ __global__ __launch_bounds__(256) void rope_cache_write_token_kernel(
       // the eight tokens' blocks share the (kv head, channel) pairs among them, an eighth each
       typedef act_t av8 __attribute__((ext_vector_type(8)));
       const size_t page0 = slot0 / bs, off0 = slot0 % bs;
-      const act_t* row0 = qkv + (size_t)tl * (nh + 2 * nkv) * hd;
+      const size_t row0 = (size_t)tl * width;
       const int items = nkv * hd, mine = (items + 7) / 8, first = (t - tl) * mine;
       for (int it = first + tid; it < min(first + mine, items); it += 256) {
         const int kvh = it / hd, d = it % hd;
-        const act_t* src = row0 + (size_t)(nh + nkv + kvh) * hd + d;
+        const size_t src = row0 + (size_t)(nh + nkv + kvh) * hd + d;
         av8 v;
 #pragma unroll
-        for (int e = 0; e < 8; e++) v[e] = src[(size_t)e * (nh + 2 * nkv) * hd];
+        for (int e = 0; e < 8; e++) v[e] = from_f32<act_t>(from.at(src + (size_t)e * width));
         *(av8*)(vcache + ((page0 * nkv + kvh) * (size_t)hd + d) * bs + off0) = v;
       }
       return;
@@ -570,14 +606,13 @@ __global__ __launch_bounds__(256) void rope_cache_write_token_kernel(
   if (slot < 0) return;
   for (int it = tid; it < nkv * (hd / 4); it += 256) {
     const int kvh = it / (hd / 4), d = (it % (hd / 4)) * 4;
-    const act_t* src = row + (size_t)(nh + nkv + kvh) * hd + d;
+    float v[4];
+    from.at4(row_at + (size_t)(nh + nkv + kvh) * hd + d, v);
     if (v_transposed) {
       act_t* vt = vcache + ((page * nkv + kvh) * (size_t)hd + d) * bs + off;
 #pragma unroll
-      for (int e = 0; e < 4; e++) vt[(size_t)e * bs] = src[e];
+      for (int e = 0; e < 4; e++) vt[(size_t)e * bs] = from_f32<act_t>(v[e]);
     } else {
-      float v[4];
-      load4<act_t>(src, v);
       store4(vcache + ((page * nkv + kvh) * bs + off) * hd + d, v);
     }
   }
@@ -797,28 +832,39 @@ int zk_softcap(float* z, size_t n, float cap, void* stream) {
   return zk_launch_status("zk_softcap");
 }
 
-int zk_rope_cache_write(void* qkv, const int* positions, const int* slot_map, const float* inv_freq,
-                        int rotary_dim, void* kcache, void* vcache, int T, int nh, int nkv, int hd,
-                        int bs, int v_transposed, void* stream) {
-  ZK_REQUIRE(T >= 0 && nh > 0 && nkv >= 0 && hd > 0 && bs > 0, "zk_rope_cache_write: bad sizes");
+// sums > 0: the rows are not in qkv yet but come as that many planes of [T, (nh + 2 nkv) hd] float
+// partial sums (a product that split K and left the adding up to its reader, see QkvSource).
+int zk_rope_cache_write_sums(void* qkv, const float* planes, int sums, const int* positions, const int* slot_map,
+                             const float* inv_freq, int rotary_dim, void* kcache, void* vcache, int T, int nh,
+                             int nkv, int hd, int bs, int v_transposed, void* stream) {
+  ZK_REQUIRE(T >= 0 && nh > 0 && nkv >= 0 && hd > 0 && bs > 0 && sums >= 0, "zk_rope_cache_write: bad sizes");
   ZK_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && rotary_dim % 2 == 0,
              "zk_rope_cache_write: rotary_dim must be even and at most head_dim");
   ZK_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "zk_rope_cache_write: no frequency table");
   ZK_REQUIRE(nh + 2 * nkv <= 65535, "zk_rope_cache_write: too many heads");
+  ZK_REQUIRE(sums == 0 || (planes != nullptr && (uintptr_t)planes % 16 == 0), "zk_rope_cache_write: partial sums must be 16-byte aligned");
   if (T == 0) return 0;
+  const QkvSource from{(const act_t*)qkv, planes, sums, (size_t)T * (nh + 2 * nkv) * hd};
   // a block a token pays off with many tokens (13.6 against 18.6 us at 2048 tokens of 8 + 2 x 4
   // heads of 256); a handful of decoded tokens is quicker spread over a block per (token, head)
   if (T >= 64 && rotary_dim == hd && hd % 8 == 0 && hd / 2 <= ROPE_MAX_HALF) {
-    rope_cache_write_token_kernel<<<T, 256, 0, (hipStream_t)stream>>>((act_t*)qkv, positions, slot_map, inv_freq,
+    rope_cache_write_token_kernel<<<T, 256, 0, (hipStream_t)stream>>>((act_t*)qkv, from, positions, slot_map, inv_freq,
                                                                      (act_t*)kcache, (act_t*)vcache, nh, nkv,
                                                                      hd, bs, v_transposed);
     return zk_launch_status("zk_rope_cache_write");
   }
   dim3 grid(T, nh + 2 * nkv);
-  rope_cache_write_kernel<<<grid, 64, 0, (hipStream_t)stream>>>((act_t*)qkv, positions, slot_map, inv_freq,
+  rope_cache_write_kernel<<<grid, 64, 0, (hipStream_t)stream>>>((act_t*)qkv, from, positions, slot_map, inv_freq,
                                                                 rotary_dim, (act_t*)kcache,
                                                                 (act_t*)vcache, nh, nkv, hd, bs, v_transposed);
   return zk_launch_status("zk_rope_cache_write");
+}
+
+int zk_rope_cache_write(void* qkv, const int* positions, const int* slot_map, const float* inv_freq,
+                        int rotary_dim, void* kcache, void* vcache, int T, int nh, int nkv, int hd,
+                        int bs, int v_transposed, void* stream) {
+  return zk_rope_cache_write_sums(qkv, nullptr, 0, positions, slot_map, inv_freq, rotary_dim, kcache, vcache, T, nh, nkv,
+                                  hd, bs, v_transposed, stream);
 }
 
 // dst_kind: 0 = float32, 1 = the library's activation type

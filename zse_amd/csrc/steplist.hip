@@ -35,6 +35,9 @@ int zk_softcap(float* z, size_t n, float cap, void* stream);
 int zk_rope_cache_write(void* qkv, const int* positions, const int* slot_map, const float* inv_freq, int rotary_dim,
                         void* kcache, void* vcache, int T, int nh, int nkv, int hd, int bs, int v_transposed,
                         void* stream);
+int zk_rope_cache_write_sums(void* qkv, const float* planes, int sums, const int* positions, const int* slot_map,
+                             const float* inv_freq, int rotary_dim, void* kcache, void* vcache, int T, int nh,
+                             int nkv, int hd, int bs, int v_transposed, void* stream);
 int zk_zero(void* p, size_t nbytes, void* stream);
 int zk_gemm_plain(const void* A, int lda, const void* W, void* C, int ldc, int c_is_f32, int M, int N, int K,
                   void* stream);
@@ -120,6 +123,7 @@ const int entered_at_load = []() {
   OWN(zk_gated_act);
   OWN(zk_softcap);
   OWN(zk_rope_cache_write);
+  OWN(zk_rope_cache_write_sums);
   OWN(zk_zero);
   OWN(zk_gemm_plain);
   OWN(zk_attention_plain);

@@ -123,7 +123,11 @@ class PagedAttention(Part):
                                cache.v.ptr, nh, n_store, hd, g.page_size, 1 if cache.v_transposed else 0,
                                ctx.stream)
         else:
-            qkv = linear(ctx, x, self.w_qkv, ctx.alloc((T, width)))
+            # a product that splits K may leave the adding up of its partial sums to the kernel
+            # that rotates and stores, unless something has to look at the rows in between
+            direct = not hooked and tables is not None and k.has("zk_rope_cache_write_sums")
+            qkv = ctx.alloc((T, width))
+            got = linear(ctx, x, self.w_qkv, qkv, sums_ok=direct)
             if hooked:
                 self.between_product_and_rotation(ctx, qkv)
             if tables is None:
@@ -131,9 +135,12 @@ class PagedAttention(Part):
                 inv_freq, rotary_dim = 0, 0
             else:
                 inv_freq, rotary_dim = tables[0].ptr, tables[1]
-            k.zk_rope_cache_write(qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map,
-                                  inv_freq or None, rotary_dim, cache.k.ptr, cache.v.ptr, T, nh, n_store,
-                                  hd, g.page_size, 1 if cache.v_transposed else 0, ctx.stream)
+            args = (ctx.positions, None if self.shared_kv else g.slot_map, inv_freq or None, rotary_dim, cache.k.ptr,
+                    cache.v.ptr, T, nh, n_store, hd, g.page_size, 1 if cache.v_transposed else 0, ctx.stream)
+            if got.layout == "parts":
+                k.zk_rope_cache_write_sums(qkv.ptr, got.ptr, got.shape[0], *args)
+            else:
+                k.zk_rope_cache_write(qkv.ptr, *args)
         o = ctx.alloc((T, nh * hd))
         cap = float(s.softcap) if s.softcap else 0.0
         win = int(s.window) if s.window else 0

@@ -15,7 +15,8 @@ def tuned_gemm(ctx, K: int) -> bool:
     return ctx.dtype == BF16 and ctx.tuned and ctx.k.has("zk_gemm_bf16") and K % 8 == 0
 
 
-def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0.0, last_of=None) -> Tensor:
+def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0.0, last_of=None,
+           sums_ok: bool = False) -> Tensor:
     """out[M, N] = x[M, K] @ w[N, K]^T with float accumulation.
 
     ``out`` may be float32 (logits) or the activation type.  In the 32-bit
@@ -30,7 +31,8 @@ def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0
     blocks, the joining launch is left out: what comes back is a float32 tensor [P, M, N] with
     layout "parts" in the product's workspace instead of ``out``, to be read before the next
     product.  A part that another part calls is not the one the block named, so it never
-    hands partial sums to a caller that does not expect them.
+    hands partial sums to a caller that does not expect them.  ``sums_ok``: the caller reads
+    such a tensor itself, whoever called it.
     """
     M, K = x.shape
     gated = epilogue in ("gelu_tanh", "silu")
@@ -52,7 +54,7 @@ def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0
         raise ValueError("linear: weights in strip layout need the matrix-core product")
     if tuned_gemm(ctx, K):
         ws = getattr(ctx, "gemm_workspace", None)      # lets a product of few columns split K over blocks
-        welcome = last_of is not None and getattr(ctx, "sums_welcome", None) is last_of
+        welcome = sums_ok or (last_of is not None and getattr(ctx, "sums_welcome", None) is last_of)
         parts = ctypes.c_int(0) if (welcome and ws is not None) else None
         k.zk_gemm_bf16(x.ptr, K, w.ptr, out.ptr, N, out_f32, M, N, K, EPILOGUES[epilogue], float(cap),
                        1 if strip else 0, ws.ptr if ws is not None else None,

@@ -148,6 +148,7 @@ KERNEL_SIGNATURES = {
     "zk_gated_act": [_VP, _VP, _I, _I, _I, _VP],
     "zk_softcap": [_VP, _SZ, _F, _VP],
     "zk_rope_cache_write": [_VP, _VP, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_rope_cache_write_sums": [_VP, _VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
     "zk_convert": [_VP, _I, _VP, _I, _SZ, _VP],
     "zk_fill_normal": [_VP, _I, _SZ, _U64, _U64, _F, _F, _VP],
     "zk_zero": [_VP, _SZ, _VP],
