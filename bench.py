@@ -442,6 +442,9 @@ def main():
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="profiling aid: run one of the two workloads (the JSON line then lacks the other)")
     ap.add_argument("--page-size", type=int, default=16, help="tokens a page of the cache holds")
+    ap.add_argument("--drawn", action="store_true",
+                    help="profiling aid: every timed decode step draws its tokens with the reference's default "
+                         "sampling parameters instead of taking the largest logit")
     ap.add_argument("--quick", action="store_true",
                     help="the headline alone: no decode at context 8,192, no 9B and 27B figures")
     a = ap.parse_args()
@@ -510,7 +513,7 @@ def main():
     for B in points:
         k = a.steps if B == a.batch else max(16, a.steps // 2)
         w = a.warmup if B == a.batch else max(4, a.warmup // 2)
-        results[B] = t.decode(B, k, w)
+        results[B] = t.decode(B, k, w, drawn=REFERENCE_SAMPLING if a.drawn else None)
         log(f"decode batch {B}: {results[B][0]:.1f} tok/s, {results[B][1] * 1e3:.3f} ms/step, "
             f"{results[B][2] / results[B][1] / 1e9:.0f} GB/s ({results[B][3]})")
     # the same at the reference's default sampling parameters (orchestrator/engine.py:40-43)
@@ -528,6 +531,7 @@ def main():
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": dict(shape_of(cfg, full_layers), model=f"gemma2-{a.model}-shapes-random", global_batch=a.batch,
+                       sampling="reference defaults" if a.drawn else "greedy",
                        seq_len=a.context, prompt_len=a.prefill_tokens, page_size=a.page_size, parallelism="single-gpu",
                        graphs=int(not a.no_graphs), graph_max_batch=graph_max_batch),
         "prefill": prefill,
