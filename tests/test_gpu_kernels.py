@@ -1185,6 +1185,14 @@ def test_the_two_ways_to_the_cut_offs(rt):
     grid = (np.round(spread * 80) / 80).astype(np.float32)      # some hundred equal logits at the cut-off
     cases.append((grid, dict(top_p=0.8), 3))
     cases.append((grid, dict(top_k=3000), 3))
+    zeros = grid.copy(); zeros[np.abs(zeros) < 0.2] = 0.0; zeros[::3] *= -1.0        # 0.0 and -0.0 are equal logits
+    assert np.signbit(zeros[zeros == 0]).any() and not np.signbit(zeros[zeros == 0]).all()
+    def share_inside_the_zeros(row):          # a share that is reached among the equal logits at zero (and by no whole number of them)
+        w = np.exp(row.astype(np.float64) / 0.8)
+        return float((w[row > 0].sum() + 0.41373 * w[row == 0].sum()) / w.sum())
+    cases.append((zeros, dict(top_p=share_inside_the_zeros(zeros)), 2))
+    few = zeros.copy(); few[1500:] -= 30.0
+    cases.append((few, dict(top_p=share_inside_the_zeros(few)), 1))
     flat = np.zeros(V, np.float32)
     cases.append((flat, dict(top_k=10), 2))
     cases.append((flat, dict(top_p=0.5005), 2))

@@ -90,14 +90,14 @@ __device__ __forceinline__ float row_max(const float* pv, int r) {
 }
 
 // Thread t of block (slice, row) owns the contiguous piece [b + t seg, b + (t + 1) seg) of the slice.
-__device__ __forceinline__ bool has_cut_offs(const int* top_k, const float* top_p, int row, int V) {
+__device__ __forceinline__ bool has_cut_offs(const int* top_k, const double* top_p, int row, int V) {
   const int k = top_k ? top_k[row] : 0;
-  return (k > 0 && k < V) || (top_p && top_p[row] < 1.f);
+  return (k > 0 && k < V) || (top_p && top_p[row] < 1.0);
 }
 
 __global__ __launch_bounds__(256) void sample_slice_sums_kernel(
     const float* __restrict__ logits, int V, const float* __restrict__ temperature, const float* __restrict__ pv,
-    const int* __restrict__ top_k, const float* __restrict__ top_p, double* __restrict__ psum) {
+    const int* __restrict__ top_k, const double* __restrict__ top_p, double* __restrict__ psum) {
   __shared__ double red[256];
   const int row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
   if (has_cut_offs(top_k, top_p, row, V)) return;
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void sample_slice_sums_kernel(
 
 __global__ __launch_bounds__(256) void sample_pick_kernel(
     const float* __restrict__ logits, int V, const float* __restrict__ temperature, const double* __restrict__ uniform,
-    const float* __restrict__ pv, const int* __restrict__ top_k, const float* __restrict__ top_p,
+    const float* __restrict__ pv, const int* __restrict__ top_k, const double* __restrict__ top_p,
     const double* __restrict__ psum, int* __restrict__ out) {
   __shared__ double red[256];
   __shared__ int s_owner;
@@ -223,8 +223,10 @@ __global__ __launch_bounds__(256) void sample_pick_kernel(
 //     narrows a range of keys (the logits' bits, made to sort like the numbers) by eight bits
 //     a pass over the whole row, four passes for top-k and four for top-p, then draws over the row;
 // A row without cut-offs (way 0) is left alone: zk_sample draws it.
+// (the two zeros are one key: they are equal logits, and which of the equal ones are kept goes
+// by their indices)
 __device__ __forceinline__ unsigned int key_of(float v) {
-  const unsigned int b = __float_as_uint(v);
+  const unsigned int b = v == 0.f ? 0u : __float_as_uint(v);
   return v != v ? 0u : ((b & 0x80000000u) ? ~b : (b | 0x80000000u));
 }
 __device__ __forceinline__ float value_of(unsigned int k) {
@@ -267,12 +269,12 @@ __device__ __forceinline__ int top_bucket(float z, float mx, float inv_t) {
   const float x = (mx - z) * inv_t;
   return x < (TOP_BUCKETS - 1) / TOP_PER_UNIT ? (int)(x * TOP_PER_UNIT) : TOP_BUCKETS - 1;
 }
-__device__ __forceinline__ void cut_kind(const int* top_k, const float* top_p, int row, int V, int& k, float& p,
+__device__ __forceinline__ void cut_kind(const int* top_k, const double* top_p, int row, int V, int& k, double& p,
                                          bool& by_count, bool& by_weight) {
   k = top_k ? top_k[row] : 0;
-  p = top_p ? top_p[row] : 1.f;
+  p = top_p ? top_p[row] : 1.0;
   by_count = k > 0 && k < V;
-  by_weight = p < 1.f;
+  by_weight = p < 1.0;
 }
 
 // f(value, index) for every NT-th element of z[b, e) from b + threadIdx.x on.  Eight loads are
@@ -293,13 +295,13 @@ __device__ __forceinline__ void each_of(const float* __restrict__ z, int b, int 
 __global__ __launch_bounds__(256) void top_hist_kernel(const float* __restrict__ logits, int V,
                                                        const float* __restrict__ pv,
                                                        const float* __restrict__ temperature,
-                                                       const int* __restrict__ top_k, const float* __restrict__ top_p,
+                                                       const int* __restrict__ top_k, const double* __restrict__ top_p,
                                                        TopRow* __restrict__ rows) {
   __shared__ unsigned int h_cnt[TOP_BUCKETS];
   __shared__ unsigned long long h_w[TOP_BUCKETS];
   const int row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
   int k;
-  float p;
+  double p;
   bool by_count, by_weight;
   cut_kind(top_k, top_p, row, V, k, p, by_count, by_weight);
   if (!by_count && !by_weight) return;
@@ -335,7 +337,7 @@ __global__ __launch_bounds__(256) void top_hist_kernel(const float* __restrict__
 __global__ __launch_bounds__(CUT_THREADS) void top_walk_kernel(const float* __restrict__ pv,
                                                                const float* __restrict__ temperature,
                                                                const int* __restrict__ top_k,
-                                                               const float* __restrict__ top_p, int V,
+                                                               const double* __restrict__ top_p, int V,
                                                                TopRow* __restrict__ rows) {
   __shared__ unsigned int c[TOP_BUCKETS];
   __shared__ unsigned long long w[TOP_BUCKETS];
@@ -343,7 +345,7 @@ __global__ __launch_bounds__(CUT_THREADS) void top_walk_kernel(const float* __re
   const int row = blockIdx.x, t = threadIdx.x;
   TopRow& tr = rows[row];
   int k;
-  float p;
+  double p;
   bool by_count, by_weight;
   cut_kind(top_k, top_p, row, V, k, p, by_count, by_weight);
   if (t == 0) {
@@ -373,7 +375,7 @@ __global__ __launch_bounds__(CUT_THREADS) void top_walk_kernel(const float* __re
     mine = c[t] >= (unsigned int)k && (t == 0 || c[t - 1] < (unsigned int)k);
   } else {
     const unsigned long long total = w[TOP_BUCKETS - 1];
-    target = (unsigned long long)ceil((double)p * (double)total);
+    target = (unsigned long long)ceil(p * (double)total);
     if (t == 0) tr.total = total;
     mine = total > 0 && w[t] >= target && (t == 0 || w[t - 1] < target);
   }
@@ -498,7 +500,7 @@ struct CutSearch {
 // from the keys that bucket holds, with what lies above it already counted, and its keys
 // spread evenly over the first pass's counters (a search from all keys puts a flat row's
 // logits into a handful of them, and the lanes of a wave wait for each other there).
-__device__ void search_row(const float* __restrict__ z, int V, float mx, float inv_t, int k, float p, bool by_count,
+__device__ void search_row(const float* __restrict__ z, int V, float mx, float inv_t, int k, double p, bool by_count,
                            bool by_weight, const TopRow* from, unsigned int* h_cnt, unsigned long long* h_w,
                            unsigned int* cnt, unsigned long long* w, CutSearch* cs, float& keep_from, int& keep_ties) {
   const int tid = threadIdx.x, wave = tid >> 6;
@@ -569,7 +571,7 @@ __device__ void search_row(const float* __restrict__ z, int V, float mx, float i
         if (weigh && cs->passes == 0) {      // the first pass covers everything top-k left: its sum is the whole
           unsigned long long total = 0;
           for (int b = 0; b < 256; b++) total += w[b];
-          cs->target = (unsigned long long)ceil((double)p * (double)total);
+          cs->target = (unsigned long long)ceil(p * (double)total);
         }
         unsigned long long acc = cs->above;
         int pick = -1, lowest = -1;
@@ -773,7 +775,7 @@ __device__ int draw_row(const float* __restrict__ z, int V, float mx, double inv
 #define CUT_LDS_BYTES (CUT_WAVES * 256 * 12 + 256 * 12 + 64)
 __global__ __launch_bounds__(CUT_THREADS) void sample_cut_kernel(
     const float* __restrict__ logits, int V, const float* __restrict__ temperature, const double* __restrict__ uniform,
-    const int* __restrict__ top_k, const float* __restrict__ top_p, TopRow* __restrict__ rows,
+    const int* __restrict__ top_k, const double* __restrict__ top_p, TopRow* __restrict__ rows,
     const Candidate* __restrict__ cand, int* __restrict__ out) {
   // ways 1 and 3: keys [TOP_CAP] and sums [TOP_CAP] of 8 bytes; way 2: the histograms
   __shared__ __attribute__((aligned(16))) unsigned char lds[CUT_LDS_BYTES > TOP_CAP * 16 ? CUT_LDS_BYTES : TOP_CAP * 16];
@@ -782,7 +784,7 @@ __global__ __launch_bounds__(CUT_THREADS) void sample_cut_kernel(
   const int row = blockIdx.x, tid = threadIdx.x;
   TopRow& tr = rows[row];
   int k;
-  float p;
+  double p;
   bool by_count, by_weight;
   cut_kind(top_k, top_p, row, V, k, p, by_count, by_weight);
   const int mode = tr.mode;
@@ -819,7 +821,7 @@ __global__ __launch_bounds__(CUT_THREADS) void sample_cut_kernel(
       __syncthreads();
       running_sums<unsigned long long>(sums, n2, nt);
       const unsigned long long total = by_count ? sums[n_k - 1] : tr.total;
-      const unsigned long long target = (unsigned long long)ceil((double)p * (double)total);
+      const unsigned long long target = (unsigned long long)ceil(p * (double)total);
       for (int i = tid; i < n_k; i += nt)
         if (sums[i] >= target && (i == 0 || sums[i - 1] < target)) s_int[1] = i + 1;
     }
@@ -928,7 +930,7 @@ size_t zk_sample_scratch_bytes(int rows) { return (size_t)rows * AM_SLICES * (8 
 
 // top_k, top_p (may be null): rows that have cut-offs (as zk_sample_cut reads them) are left alone.
 int zk_sample(const float* logits, const float* temperature, const double* uniform, const int* top_k,
-              const float* top_p, int* out, int rows, int V, void* scratch, void* stream) {
+              const double* top_p, int* out, int rows, int V, void* scratch, void* stream) {
   ZK_REQUIRE(rows >= 0 && V > 0, "zk_sample: bad sizes");
   ZK_REQUIRE(rows <= 65535, "zk_sample: too many rows");
   ZK_REQUIRE(scratch != nullptr && (uintptr_t)scratch % 8 == 0, "zk_sample: no scratch buffer");
@@ -956,7 +958,7 @@ size_t zk_sample_cut_row_bytes() { return sizeof(TopRow); }
 size_t zk_sample_cut_mode_offset() { return offsetof(TopRow, mode); }
 
 int zk_sample_cut(const float* logits, const float* temperature, const double* uniform, const int* top_k,
-                  const float* top_p, int* out, int rows, int V, void* scratch, int room, void* stream) {
+                  const double* top_p, int* out, int rows, int V, void* scratch, int room, void* stream) {
   ZK_REQUIRE(rows >= 0 && V > 0 && room >= rows, "zk_sample_cut: bad sizes");
   ZK_REQUIRE(rows <= 65535, "zk_sample_cut: too many rows");
   ZK_REQUIRE(temperature && uniform && out, "zk_sample_cut: temperature, uniform numbers and output are needed");

@@ -150,16 +150,16 @@ class DeviceSampler:
         self.scratch = rt.empty(((kernels.zk_sample_scratch_bytes(max_rows) + 3) // 4,), F32)
         self.cut_scratch = None                             # histograms and candidates of the cut-offs, on first use
         self.top_k = rt.empty((max_rows,), I32)
-        self.top_p = rt.empty((max_rows,), F32)
+        self.top_p = rt.empty((max_rows,), F64)
         self._pen = None                                    # (rows, tokens, scales) on the device, grown on demand
         # the rows' temperatures, uniform numbers and cut-offs on their way to the device: page-locked,
         # so their copies queue behind the step's kernels instead of waiting for them (``sample``
         # reads its ids before it returns, so the next call finds the buffer free)
-        self._stage = rt.pinned(max_rows * 20)
+        self._stage = rt.pinned(max_rows * 24)
         self._stage_u = self._stage.array(0, max_rows, np.float64)
-        self._stage_t = self._stage.array(max_rows * 8, max_rows, np.float32)
-        self._stage_k = self._stage.array(max_rows * 12, max_rows, np.int32)
-        self._stage_p = self._stage.array(max_rows * 16, max_rows, np.float32)
+        self._stage_p = self._stage.array(max_rows * 8, max_rows, np.float64)
+        self._stage_t = self._stage.array(max_rows * 16, max_rows, np.float32)
+        self._stage_k = self._stage.array(max_rows * 20, max_rows, np.int32)
 
     # ---- a run of steps without waiting for the host in between
     RING = 16       # results that may be on their way to the host at a time
@@ -202,7 +202,7 @@ class DeviceSampler:
         self._run_plain = any(self._is_plain(r["params"], vocab) for r in rows)
         if self._run_cut:
             self.rt.copy_h2d(self.top_k.ptr, np.array([r["params"].top_k for r in rows], dtype=np.int32))
-            self.rt.copy_h2d(self.top_p.ptr, np.array([r["params"].top_p for r in rows], dtype=np.float32))
+            self.rt.copy_h2d(self.top_p.ptr, np.array([r["params"].top_p for r in rows], dtype=np.float64))
         flat = np.ascontiguousarray(np.asarray(us, dtype=np.float64).reshape(len(us), n))
         if getattr(self, "_run_u", None) is None or self._run_u.shape[0] < flat.size:
             self._run_u = self.rt.empty((max(flat.size, self.max_rows * 8),), F64)
@@ -259,7 +259,7 @@ class DeviceSampler:
             st = self._stage.ptr
             self._stage_t[:n] = [1.0 if g else r["params"].temperature for r, g in zip(rows, greedy)]
             self._stage_u[:n] = [r["u"] for r in rows]
-            rt.copy_h2d_async(self.temp.ptr, st + self.max_rows * 8, n * 4)
+            rt.copy_h2d_async(self.temp.ptr, st + self.max_rows * 16, n * 4)
             rt.copy_h2d_async(self.u.ptr, st, n * 8)
             cut = any(not g and self._has_cut(r["params"], V) for r, g in zip(rows, greedy))
             plain = any(not g and self._is_plain(r["params"], V) for r, g in zip(rows, greedy))
@@ -267,8 +267,8 @@ class DeviceSampler:
                 # (a greedy row, whose draw nobody reads, as top-k 1: the cheapest there is)
                 self._stage_k[:n] = [1 if g else r["params"].top_k for r, g in zip(rows, greedy)]
                 self._stage_p[:n] = [1.0 if g else r["params"].top_p for r, g in zip(rows, greedy)]
-                rt.copy_h2d_async(self.top_k.ptr, st + self.max_rows * 12, n * 4)
-                rt.copy_h2d_async(self.top_p.ptr, st + self.max_rows * 16, n * 4)
+                rt.copy_h2d_async(self.top_k.ptr, st + self.max_rows * 20, n * 4)
+                rt.copy_h2d_async(self.top_p.ptr, st + self.max_rows * 8, n * 8)
             self._draw(logits, n, V, self.u.ptr, cut, plain)
         g = rt.download(self.ids.rows(0, n)) if any(greedy) else None
         s = rt.download(self.ids2.rows(0, n)) if not all(greedy) else None
