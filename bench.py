@@ -174,7 +174,6 @@ def check_decode_path(model, rt, vocab, B, use_graphs):
                 ids.append(z.argmax(axis=1).tolist())
         else:
             sampler = DeviceSampler(rt, runner.k, B)
-            sampler.prepare_run([{"params": SamplingParams(temperature=0.0), "u": 0.0} for _ in range(B)], [[0.0] * B])
             fed, pending = None, []
             for _ in range(n_steps):
                 toks = ids[0] if fed is None else [0] * B
@@ -349,17 +348,17 @@ class Timed:
         # its logits to the sampling kernels; either way the ids stay on the device, the next step
         # takes them from there, and the host reads them four steps at a time (it has to, for stop
         # tokens) while the next steps are already enqueued.
-        us = rng.random((4, B)).tolist()
-        sampler.prepare_run(rows, us, vocab=V)
-        pending, fed, turn = [], None, 0
+        pending, fed = [], None
 
         def one():
-            nonlocal fed, turn
+            nonlocal fed
             toks = first if fed is None else [0] * B
             entries = [StepEntry(r, [t], [0]) for r, t in zip(reqs, toks)]
             if drawn:
-                ids = sampler.sample_deferred(runner.step(entries, download=False, tokens_from=fed), turn % 4)
-                turn += 1
+                for row in rows:
+                    row["u"] = float(rng.random())
+                staged = sampler.stage(rows, V)
+                ids = sampler.sample_staged(runner.step(entries, download=False, tokens_from=fed), staged)
             else:
                 ids = sampler.ids_deferred(runner.step(entries, download=False, tokens_from=fed, pick=True))
             fed = ids.device_ptr

@@ -350,3 +350,82 @@ def test_the_windowed_group_gets_a_pool_of_its_own_size(tiny_folders):
     for p, g in zip(prompts, got):
         assert g == plain_greedy(cfg, w, p, 20)
     eng.close()
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tokens_fed_on_the_device_to_any_entries_of_a_step(tiny_folders, dtype, graphs):
+    """A step takes the tokens of some of its entries from the ids the step before left on the
+    device, whatever the order of the entries, beside a portion of a prompt that brings its
+    own tokens: the same logits, to the bit, as when the host brings those tokens."""
+    from gpu_util import make_runner
+    from zse_amd.engine.runner import StepEntry
+    from zse_amd.sampling import DeviceSampler, SamplingParams
+    cfg = TINY["A"][0]
+    folder = tiny_folders[("A", dtype)]
+    V = cfg["vocab_size"]
+    prompts = {r: random_tokens(V, n, 30 + n) for r, n in (("a", 9), ("b", 4), ("c", 13), ("d", 21))}
+
+    def run(on_device):
+        runner = make_runner(folder, dtype, max_seqs=8, use_graphs=graphs)
+        sampler = DeviceSampler(runner.rt, runner.k, 8)
+        greedy = [{"params": SamplingParams(temperature=0.0), "u": 0.0} for _ in range(3)]
+        logits = runner.step([StepEntry(r, prompts[r], [len(prompts[r]) - 1]) for r in "abc"], download=False)
+        ids = sampler.sample_staged(logits, sampler.stage(greedy, V))
+        host = ids.result()
+        out = []
+        # b and a decode in another order than they were sampled in, c sits the step out, d arrives with a portion
+        entries = [StepEntry("d", prompts["d"][:12], []), StepEntry("b", [0 if on_device else host[1]], [0]),
+                   StepEntry("a", [0 if on_device else host[0]], [0])]
+        if on_device:
+            out.append(runner.step(entries, tokens_from=ids.device_ptr, feed=[-1, 1, 0]))
+        else:
+            out.append(runner.step(entries))
+        # and a step of single tokens through a graph or a launch list, fed in another order again
+        logits = runner.step([StepEntry("a", [5], [0]), StepEntry("b", [6], [0]), StepEntry("c", [host[2]], [0])], download=False)
+        ids = sampler.sample_staged(logits, sampler.stage(greedy, V))
+        host = ids.result()
+        entries = [StepEntry("c", [0 if on_device else host[2]], [0]), StepEntry("a", [0 if on_device else host[0]], [0]),
+                   StepEntry("d", prompts["d"][12:14], [1])]
+        out.append(runner.step(entries, tokens_from=ids.device_ptr, feed=[2, 0, -1]) if on_device else runner.step(entries))
+        entries = [StepEntry(r, [7], [0]) for r in "cab"]
+        logits = runner.step(entries, download=False)
+        ids = sampler.sample_staged(logits, sampler.stage(greedy, V))
+        host = ids.result()
+        entries = [StepEntry("b", [0 if on_device else host[2]], [0]), StepEntry("c", [0 if on_device else host[0]], [0])]
+        out.append(runner.step(entries, tokens_from=ids.device_ptr, feed=[2, 0]) if on_device else runner.step(entries))
+        runner.close()
+        return out
+
+    for got, want in zip(run(True), run(False)):
+        assert got.shape == want.shape and np.array_equal(got, want)
+    with pytest.raises(ValueError):
+        runner = make_runner(folder, dtype, max_seqs=8)
+        try:
+            runner.step([StepEntry("a", [1, 2], [1])], tokens_from=1, feed=[0])
+        finally:
+            runner.close()
+
+
+def test_a_stream_of_tokens_never_shows_a_placeholder(tiny_folders):
+    """``stream_generate_tokens`` and ``step`` hand out tokens the host has seen; ``run`` reads the
+    ids some steps behind the steps it enqueues and ends with the same outputs."""
+    from zse_amd.engine.engine import Engine
+    from zse_amd.sampling import SamplingParams
+    cfg = TINY["B"][0]
+    folder = tiny_folders[("B", "float32")]
+    prompts = [random_tokens(cfg["vocab_size"], n, 170 + n) for n in (5, 12, 3)]
+    eng = Engine(folder, dtype="float32", block_size=8, max_batch_tokens=32, max_batch_seqs=4, prefill_chunk_size=7,
+                 max_seq_len=128, decode_run=4)
+    kw = dict(max_tokens=19, temperature=0.8, top_k=20, seed=5)
+    streamed = list(eng.stream_generate_tokens(prompts[0], **kw))
+    assert len(streamed) == 19 and all(0 <= t < cfg["vocab_size"] for t in streamed)
+    assert eng.generate([prompts[0]], SamplingParams(**kw))[0] == streamed
+    params = [SamplingParams(max_tokens=m, temperature=t, seed=9 + i) for i, (m, t) in enumerate(((15, 0.0), (9, 1.1), (22, 0.7)))]
+    by_run = eng.generate(prompts, params)
+    reqs = [eng.add_request(p, sp) for p, sp in zip(prompts, params)]
+    while eng.scheduler.has_work():
+        eng.step()
+        assert all(-1 not in r.output_tokens for r in reqs)
+    assert [list(r.output_tokens) for r in reqs] == by_run
+    eng.close()

@@ -618,6 +618,12 @@ __global__ __launch_bounds__(256) void rope_cache_write_token_kernel(
   }
 }
 
+__global__ void feed_tokens_kernel(int* __restrict__ tokens, const int* __restrict__ ids, const int* __restrict__ dst,
+                                   const int* __restrict__ src, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) tokens[dst[i]] = ids[src[i]];
+}
+
 // ------------------------------------------------------------------ conversion, fill
 
 // src_tag: 0 = float32, 1 = bfloat16, 2 = float16
@@ -890,6 +896,17 @@ int zk_fill_normal(void* dst, int dst_kind, size_t n, uint64_t seed, uint64_t st
   if (dst_kind == 0) fill_normal_kernel<float><<<g, 256, 0, s>>>((float*)dst, n, seed, stream_id, mean, std);
   else fill_normal_kernel<act_t><<<g, 256, 0, s>>>((act_t*)dst, n, seed, stream_id, mean, std);
   return zk_launch_status("zk_fill_normal");
+}
+
+// tokens[dst[i]] = ids[src[i]] for i < n: the ids a step's sampling left on the device become
+// the next step's tokens without a trip to the host, for the requests the next step decodes, in
+// whatever order it holds them.
+int zk_feed_tokens(int* tokens, const int* ids, const int* dst, const int* src, int n, void* stream) {
+  ZK_REQUIRE(n >= 0, "zk_feed_tokens: bad count");
+  if (n == 0) return 0;
+  ZK_REQUIRE(tokens && ids && dst && src, "zk_feed_tokens: null argument");
+  feed_tokens_kernel<<<(n + 255) / 256, 256, 0, (hipStream_t)stream>>>(tokens, ids, dst, src, n);
+  return zk_launch_status("zk_feed_tokens");
 }
 
 // Clears ``nbytes`` (a multiple of 4) with a kernel, so that it may be captured in a graph.

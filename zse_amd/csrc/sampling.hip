@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void sample_slice_sums_kernel(
     const int* __restrict__ top_k, const double* __restrict__ top_p, double* __restrict__ psum) {
   __shared__ double red[256];
   const int row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
-  if (has_cut_offs(top_k, top_p, row, V)) return;
+  if (temperature[row] <= 0.f || has_cut_offs(top_k, top_p, row, V)) return;
   const float* z = logits + (size_t)row * V;
   const double inv_t = 1.0 / (double)temperature[row];
   const float mx = row_max(pv, row);
@@ -127,7 +127,7 @@ __global__ __launch_bounds__(256) void sample_pick_kernel(
   __shared__ int s_owner;
   __shared__ double s_before;
   const int row = blockIdx.x, tid = threadIdx.x;
-  if (has_cut_offs(top_k, top_p, row, V)) return;
+  if (temperature[row] <= 0.f || has_cut_offs(top_k, top_p, row, V)) return;
   const float* z = logits + (size_t)row * V;
   const double inv_t = 1.0 / (double)temperature[row];
   const float mx = row_max(pv, row);
@@ -269,12 +269,13 @@ __device__ __forceinline__ int top_bucket(float z, float mx, float inv_t) {
   const float x = (mx - z) * inv_t;
   return x < (TOP_BUCKETS - 1) / TOP_PER_UNIT ? (int)(x * TOP_PER_UNIT) : TOP_BUCKETS - 1;
 }
-__device__ __forceinline__ void cut_kind(const int* top_k, const double* top_p, int row, int V, int& k, double& p,
-                                         bool& by_count, bool& by_weight) {
+__device__ __forceinline__ void cut_kind(const float* temperature, const int* top_k, const double* top_p, int row, int V,
+                                         int& k, double& p, bool& by_count, bool& by_weight) {
   k = top_k ? top_k[row] : 0;
   p = top_p ? top_p[row] : 1.0;
-  by_count = k > 0 && k < V;
-  by_weight = p < 1.0;
+  const bool drawn = temperature[row] > 0.f;       // a row that is not drawn has no cut-offs either
+  by_count = drawn && k > 0 && k < V;
+  by_weight = drawn && p < 1.0;
 }
 
 // f(value, index) for every NT-th element of z[b, e) from b + threadIdx.x on.  Eight loads are
@@ -303,7 +304,7 @@ __global__ __launch_bounds__(256) void top_hist_kernel(const float* __restrict__
   int k;
   double p;
   bool by_count, by_weight;
-  cut_kind(top_k, top_p, row, V, k, p, by_count, by_weight);
+  cut_kind(temperature, top_k, top_p, row, V, k, p, by_count, by_weight);
   if (!by_count && !by_weight) return;
   const bool weigh = !by_count;
   for (int i = tid; i < TOP_BUCKETS; i += 256) {
@@ -347,7 +348,7 @@ __global__ __launch_bounds__(CUT_THREADS) void top_walk_kernel(const float* __re
   int k;
   double p;
   bool by_count, by_weight;
-  cut_kind(top_k, top_p, row, V, k, p, by_count, by_weight);
+  cut_kind(temperature, top_k, top_p, row, V, k, p, by_count, by_weight);
   if (t == 0) {
     tr.mx = row_max(pv, row);
     tr.inv_t = 1.f / temperature[row];
@@ -786,7 +787,7 @@ __global__ __launch_bounds__(CUT_THREADS) void sample_cut_kernel(
   int k;
   double p;
   bool by_count, by_weight;
-  cut_kind(top_k, top_p, row, V, k, p, by_count, by_weight);
+  cut_kind(temperature, top_k, top_p, row, V, k, p, by_count, by_weight);
   const int mode = tr.mode;
   if (mode == 0) return;          // no cut-offs: zk_sample's row
   const float mx = tr.mx, inv_t = tr.inv_t;
@@ -928,7 +929,9 @@ int zk_argmax(const float* logits, int* out, int rows, int V, void* scratch, voi
 // scratch: as for zk_argmax plus rows * 64 doubles (zk_sample_scratch_bytes)
 size_t zk_sample_scratch_bytes(int rows) { return (size_t)rows * AM_SLICES * (8 + 8); }
 
-// top_k, top_p (may be null): rows that have cut-offs (as zk_sample_cut reads them) are left alone.
+// top_k, top_p (may be null): rows that have cut-offs (as zk_sample_cut reads them) are left alone,
+// and so is a row whose temperature is not positive (its caller takes the largest logit: zk_argmax
+// into the same ``out`` first serves a batch of both kinds).
 int zk_sample(const float* logits, const float* temperature, const double* uniform, const int* top_k,
               const double* top_p, int* out, int rows, int V, void* scratch, void* stream) {
   ZK_REQUIRE(rows >= 0 && V > 0, "zk_sample: bad sizes");
@@ -947,7 +950,8 @@ int zk_sample(const float* logits, const float* temperature, const double* unifo
 }
 
 // Draws the rows that have top-k or top-p.  top_k[r] <= 0 or >= V: no top-k; top_p[r] >= 1: no
-// top-p; either pointer may be null; out[r] of a row with neither is not written.  scratch: zk_sample_cut_scratch_bytes(room) bytes, room >= rows, that
+// top-p; either pointer may be null; out[r] of a row with neither, or whose temperature is not
+// positive, is not written.  scratch: zk_sample_cut_scratch_bytes(room) bytes, room >= rows, that
 // held zero when they were first handed in and are handed in again, with the same room, as the
 // last call left them.
 size_t zk_sample_cut_scratch_bytes(int rows) {

@@ -11,6 +11,7 @@ Prompts are token ids: text and tokenizers are outside this engine.
 from __future__ import annotations
 
 import time
+from collections import deque
 from dataclasses import dataclass, field
 from typing import Dict, Iterator, List, Optional, Sequence, Union
 
@@ -20,7 +21,7 @@ from .loading import load_model, random_model
 from .model import Model
 from .request import FinishReason, Request, RequestState
 from .runner import StepEntry, StepRunner
-from .scheduler import Scheduler, SchedulerConfig, StepPlan
+from .scheduler import UNKNOWN_TOKEN, Scheduler, SchedulerConfig, StepPlan
 
 
 @dataclass
@@ -88,6 +89,10 @@ class Engine:
         # device; a stop token found afterwards cuts the request's output back to it.
         self.decode_run = max(1, min(int(decode_run), DeviceSampler.RING))     # results on their way at a time
         self._next_plan: Optional[StepPlan] = None
+        # steps whose ids are still on their way: (the ids, [(request, its place in the output)]);
+        # the last of them left its ids at _last_ids, the row of request r at _last_rows[r]
+        self._pending = deque()
+        self._last_ids, self._last_rows = None, {}
 
     def _pages_per_group(self, num_blocks: Optional[int], block_size: int, max_seqs: int, max_len: int,
                          step_tokens: int) -> List[int]:
@@ -131,30 +136,74 @@ class Engine:
         return req
 
     def step(self) -> List[Request]:
-        """Schedule, run and sample one step (or a run of decode steps); returns the requests
-        that finished in it."""
+        """Schedule, run and sample one step, or up to ``decode_run`` steps enqueued one behind
+        the other where that is possible (``_can_run_ahead``); every id has reached the host
+        when this returns.  Returns the requests that finished."""
         t0 = time.monotonic()
-        plan, self._next_plan = self._next_plan or self.scheduler.schedule(), None
+        plan = self._take_plan()
         if not plan:
             return list(plan.failed)
-        pools = self.runner.manager.pools
-        if len(self._stats.peak_pages) != len(pools):
-            self._stats.peak_pages = [0] * len(pools)
-        self._stats.peak_pages = [max(a, p.used_pages) for a, p in zip(self._stats.peak_pages, pools)]
-        multi = any(s.count > 1 for s in plan.items)
-        single = any(s.count == 1 and s.request.state == RequestState.DECODING for s in plan.items)
-        kind = "mixed" if multi and single else ("prefill" if multi or not single else "decode")
-        steps0, tokens = self._stats.steps, plan.num_tokens
-        done = self._step(plan)
+        kind, steps0, tokens = self._kind(plan), self._stats.steps, plan.num_tokens
+        if self._can_run_ahead(plan):
+            done = []
+            for i in range(self.decode_run):
+                done += self._enqueue(plan)
+                if i + 1 == self.decode_run:
+                    break
+                nxt = self.scheduler.schedule()
+                if not nxt or not self._can_run_ahead(nxt):
+                    self._next_plan = nxt
+                    break
+                plan = nxt
+            done += self._resolve(0)
+        else:
+            done = self._step_and_wait(plan)
         n = self._stats.steps - steps0
         self._stats.note_step(kind, n, tokens * max(n, 1), time.monotonic() - t0)
         self._stats.note_finished(done)
         return done
 
-    def _step(self, plan: StepPlan) -> List[Request]:
-        run = self._run_length(plan)
-        if run >= 2:
-            return self._decode_run(plan, run)
+    def run(self) -> None:
+        """Every request to its end.  Steps are enqueued without waiting for their ids wherever
+        ``_can_run_ahead`` allows; the ids of a step are read when ``decode_run`` later steps
+        have been enqueued behind it, so the device has work while the host reads, plans and
+        packs."""
+        t0 = time.monotonic()
+        while self.scheduler.has_work() or self._pending:
+            t1 = time.monotonic()
+            plan = self._take_plan()
+            if not plan:
+                done = self._resolve(0) + list(plan.failed)
+                self._stats.note_finished(done)
+                continue
+            kind, steps0, tokens = self._kind(plan), self._stats.steps, plan.num_tokens
+            if self._can_run_ahead(plan):
+                done = self._enqueue(plan) + self._resolve(self.decode_run - 1)
+            else:
+                done = self._resolve(0)            # the host has to see every id first
+                plan.items = [s for s in plan.items if not s.request.finished]
+                done += self._step_and_wait(plan) if plan.items else list(plan.failed)
+            self._stats.note_step(kind, self._stats.steps - steps0, tokens, time.monotonic() - t1)
+            self._stats.note_finished(done)
+        self._stats.seconds += time.monotonic() - t0
+
+    def _take_plan(self) -> StepPlan:
+        plan, self._next_plan = (self._next_plan if self._next_plan is not None else self.scheduler.schedule()), None
+        if plan:
+            pools = self.runner.manager.pools
+            if len(self._stats.peak_pages) != len(pools):
+                self._stats.peak_pages = [0] * len(pools)
+            self._stats.peak_pages = [max(a, p.used_pages) for a, p in zip(self._stats.peak_pages, pools)]
+        return plan
+
+    @staticmethod
+    def _kind(plan: StepPlan) -> str:
+        multi = any(s.count > 1 for s in plan.items)
+        single = any(s.count == 1 and s.request.state == RequestState.DECODING for s in plan.items)
+        return "mixed" if multi and single else ("prefill" if multi or not single else "decode")
+
+    def _step_and_wait(self, plan: StepPlan) -> List[Request]:
+        """One step whose ids the host reads before it goes on (nothing is on its way)."""
         entries = [StepEntry(s.request.request_id,
                              s.request.tokens_at(s.start, s.count),
                              [s.count - 1] if s.sample else []) for s in plan.items]
@@ -169,86 +218,87 @@ class Engine:
                 who.append(r.request_id)
         ids = self.sampler.sample(logits, rows) if rows else []
         done = self.scheduler.on_step_done(plan, dict(zip(who, ids)))
+        self._last_rows = {}
         self._stats.steps += 1
         self._stats.generated_tokens += len(ids)
         self._stats.preemptions = self.scheduler.num_preemptions
         return done + list(plan.failed)
 
-    # ---- several steps of single tokens without waiting for the host in between
-    def _rows(self, plan: StepPlan, ahead: int = 0) -> List[dict]:
-        return [{"params": s.request.params, "u": uniform(s.request.seed, len(s.request.output_tokens) + ahead),
+    # ---- steps that do not wait for the host
+    def _rows(self, plan: StepPlan) -> List[dict]:
+        return [{"params": s.request.params, "u": uniform(s.request.seed, len(s.request.output_tokens)),
                  "past": ()} for s in plan.items if s.sample]
 
-    def _run_length(self, plan: StepPlan) -> int:
-        """How many steps can follow each other before the host reads an id: every request
-        decodes (so whoever waits could not be admitted to this step), is sampled on the
-        device in one manner, and nobody reaches its length before the run's last step.  The
-        run ends early when a later step's plan differs, a newcomer included; a request that
-        waits only for a stop token found late waits a few steps longer."""
-        if self.decode_run < 2 or plan.preempted or plan.failed:
-            return 1
-        if not all(s.count == 1 and s.sample and s.request.state == RequestState.DECODING for s in plan.items):
-            return 1
-        if not self.sampler.can_defer(self._rows(plan)):
-            return 1
-        n = self.decode_run
+    def _can_run_ahead(self, plan: StepPlan) -> bool:
+        """Whether the plan's step may be enqueued before the ids of the steps before it have
+        reached the host: its requests are sampled on the device from nothing but their logits
+        (no repetition penalty), nothing is out of the ordinary (nobody was preempted or
+        turned away), and a token that the host has not seen yet is the one token its request
+        brings and was drawn by the step just before, whose ids are still on the device."""
+        if self.decode_run < 2 or not plan or plan.preempted or plan.failed:
+            return False
+        for s in plan.items:
+            if s.request.tokens_at(s.start + s.count - 1, 1)[0] == UNKNOWN_TOKEN and \
+                    (s.count != 1 or s.request.request_id not in self._last_rows):
+                return False
+        return self.sampler.can_defer(self._rows(plan))
+
+    def _enqueue(self, plan: StepPlan) -> List[Request]:
+        """One step, nothing awaited.  A request's token that the step before has drawn and the
+        host has not seen yet is fed to the step on the device; its place in the request's
+        output holds a placeholder until the ids arrive (``_resolve``), and the scheduler plans
+        with the numbers of tokens, which it knows.  Returns the requests that reached their
+        length."""
+        sch, runner, sampler = self.scheduler, self.runner, self.sampler
+        entries, feed = [], []
         for s in plan.items:
             r = s.request
-            n = min(n, r.params.max_tokens - len(r.output_tokens), self.runner.manager.max_model_len - r.num_tokens)
-        return n
+            toks = r.tokens_at(s.start, s.count)
+            src = -1
+            if toks[-1] == UNKNOWN_TOKEN:           # drawn by the step before, still on the device
+                src, toks = self._last_rows[r.request_id], [0]
+            entries.append(StepEntry(r.request_id, toks, [s.count - 1] if s.sample else []))
+            feed.append(src)
+        fed = any(x >= 0 for x in feed)
+        rows = self._rows(plan)
+        places = [(s.request, len(s.request.output_tokens)) for s in plan.items if s.sample]
+        staged = sampler.stage(rows, runner.vocab) if rows else None
+        kw = dict(download=False, tokens_from=self._last_ids if fed else None, feed=feed if fed else None)
+        if rows and staged["all_greedy"]:
+            # the step picks the largest logits itself (in the head product's epilogue where
+            # the kernels can: the logits then never reach memory)
+            ids = sampler.ids_deferred(runner.step(entries, pick=True, **kw))
+        else:
+            logits = runner.step(entries, **kw)
+            ids = sampler.sample_staged(logits, staged) if rows else None
+        if ids is not None:
+            self._pending.append((ids, places))
+            self._last_ids, self._last_rows = ids.device_ptr, {r.request_id: j for j, (r, _) in enumerate(places)}
+        else:
+            self._last_rows = {}
+        self._stats.steps += 1
+        return sch.on_step_done(plan, {r.request_id: None for r, _ in places})
 
-    def _decode_run(self, plan: StepPlan, length: int) -> List[Request]:
-        sch, runner, sampler = self.scheduler, self.runner, self.sampler
-        reqs = [s.request for s in plan.items]
-        first_len = [len(r.output_tokens) for r in reqs]
-        sampler.prepare_run(self._rows(plan), [[uniform(r.seed, n0 + i) for r, n0 in zip(reqs, first_len)]
-                                               for i in range(length)], vocab=runner.vocab)
-        pending, done, tokens_from = [], [], None
-        for i in range(length):
-            known = tokens_from is None
-            entries = [StepEntry(r.request_id, [r.tokens_at(s.start, 1)[0] if known else 0], [0])
-                       for r, s in zip(reqs, plan.items)]
-            if sampler.run_is_greedy:
-                # the step picks the largest logits itself (in the head product's epilogue where
-                # the kernels can: the logits then never reach memory)
-                ids = sampler.ids_deferred(runner.step(entries, download=False, tokens_from=tokens_from, pick=True))
-            else:
-                logits = runner.step(entries, download=False, tokens_from=tokens_from)
-                ids = sampler.sample_deferred(logits, i)
-            pending.append(ids)
-            tokens_from = ids.device_ptr
-            done += sch.on_step_done(plan, {r.request_id: None for r in reqs})
-            self._stats.steps += 1
-            if i + 1 == length:
-                break
-            plan = sch.schedule()
-            same = (not plan.preempted and not plan.failed and [s.request for s in plan.items] == reqs
-                    and all(s.count == 1 and s.sample for s in plan.items))
-            if not same:                       # pages ran short: look at the ids before going on
-                self._next_plan = plan
-                break
-        # the ids arrive: put them where the placeholders are, and end what a stop token ends
-        stopped = set()
-        for i, ids in enumerate(pending):
-            for r, n0, tok in zip(reqs, first_len, ids.result()):
-                if r.request_id in stopped:
+    def _resolve(self, keep: int) -> List[Request]:
+        """Reads the ids of the enqueued steps, oldest first, until at most ``keep`` steps are
+        still on their way: puts them where the placeholders are and ends what a stop token
+        ends (the request's output is cut back to it; what was computed for it since is thrown
+        away).  Returns the requests that ended so."""
+        done = []
+        while len(self._pending) > keep:
+            ids, places = self._pending.popleft()
+            for (r, at), tok in zip(places, ids.result()):
+                if at >= len(r.output_tokens):          # behind a stop token found in an earlier step
                     continue
-                r.output_tokens[n0 + i] = tok
+                r.output_tokens[at] = tok
+                self._stats.generated_tokens += 1
                 if r.params.stop_tokens and tok in r.params.stop_tokens:
-                    stopped.add(r.request_id)
-                    if sch.finish_at(r, n0 + i + 1, FinishReason.STOP):
+                    if self.scheduler.finish_at(r, at + 1, FinishReason.STOP):
                         done.append(r)
-        if self._next_plan is not None and stopped:
-            self._next_plan.items = [s for s in self._next_plan.items if s.request.request_id not in stopped]
-        self._stats.generated_tokens += sum(len(r.output_tokens) - n0 for r, n0 in zip(reqs, first_len))
-        self._stats.preemptions = sch.num_preemptions
+        if done and self._next_plan is not None:
+            self._next_plan.items = [s for s in self._next_plan.items if not s.request.finished]
+        self._stats.preemptions = self.scheduler.num_preemptions
         return done
-
-    def run(self) -> None:
-        t0 = time.monotonic()
-        while self.scheduler.has_work():
-            self.step()
-        self._stats.seconds += time.monotonic() - t0
 
     # ---- the calls users make
     def generate(self, prompts: Sequence[Sequence[int]],

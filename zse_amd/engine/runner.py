@@ -268,7 +268,7 @@ class StepRunner:
 
     # ------------------------------------------------------------------ sizes
     def _meta_words(self, T: int, R: int, G: int) -> int:
-        return 4 * T + (R + 1) + 2 * R + G * (T + R * self.max_blocks) + 64
+        return 4 * T + (R + 1) + 4 * R + G * (T + R * self.max_blocks) + 64
 
     def cache_bytes(self) -> int:
         return sum(c.k.nbytes + c.v.nbytes for c in self.caches if c.k is not None)
@@ -307,8 +307,11 @@ class StepRunner:
         self.manager.release(req)
 
     # ------------------------------------------------------------------ the step
-    def _pack(self, entries: Sequence[StepEntry], T_pad: int, R_pad: int):
-        """Fill the pinned host buffer; returns offsets (in words) and counts."""
+    def _pack(self, entries: Sequence[StepEntry], T_pad: int, R_pad: int, feed: Optional[Sequence[int]] = None):
+        """Fill the pinned host buffer; returns offsets (in words) and counts.  ``feed``: per
+        entry the place among the last step's ids that holds its token, or -1; the pairs
+        (place of the token in this step, place of the id) go to the device with the rest and
+        ``self._fed`` says how many they are."""
         m, ps = self.manager, self.page_size
         G = len(m.groups)
         T = sum(len(e.tokens) for e in entries)
@@ -329,6 +332,8 @@ class StepRunner:
         q_start = take("q_start", R_pad + 1)
         ctx_len = take("ctx_len", R_pad)
         slot_of_req = take("slot_of_req", R_pad)
+        feed_dst = take("feed_dst", R_pad)
+        feed_src = take("feed_src", R_pad)
         slot_maps = [take(f"slot_map{g}", T_pad) for g in range(G)]
         tables = [take(f"table{g}", R_pad * self.max_blocks).reshape(R_pad, self.max_blocks)
                   for g in range(G)]
@@ -383,6 +388,13 @@ class StepRunner:
                                      f"{len(e.tokens)} tokens")
                 logit_rows[n_rows] = first_token[i] + w
                 n_rows += 1
+        self._fed = 0
+        if feed is not None:
+            for i, src in enumerate(feed):
+                if src >= 0:
+                    feed_dst[self._fed] = first_token[i]
+                    feed_src[self._fed] = src
+                    self._fed += 1
         q_start[R:] = T
         ctx_len[R:] = 0
         slot_of_req[R:] = 0
@@ -452,7 +464,18 @@ class StepRunner:
             b *= 2
         return b if b <= self.max_seqs else 0
 
-    def _graph_step(self, entries, bucket: int, tokens_from=None, pick=False):
+    def _feed(self, off, tokens_from: Optional[int], R: int, identity: bool) -> None:
+        """After the step's arrays have been sent: the tokens that come from the last step's ids."""
+        if tokens_from is None:
+            return
+        if identity:
+            self.rt.copy_d2d(self.meta_dev.ptr + off["tokens"] * 4, tokens_from, R * 4)
+        elif self._fed:
+            base = self.meta_dev.ptr
+            self.k.zk_feed_tokens(base + off["tokens"] * 4, tokens_from, base + off["feed_dst"] * 4,
+                                  base + off["feed_src"] * 4, self._fed, self.rt.stream)
+
+    def _graph_step(self, entries, bucket: int, tokens_from=None, pick=False, feed=None):
         """One token for each request through a graph of this bucket.  The first step of
         a bucket runs eagerly (it sizes the arena), later ones are captured and replayed.
         Kernel arguments are fixed by the graph: rows beyond the batch are padding (position
@@ -463,7 +486,7 @@ class StepRunner:
         attention kernels' grids; a block past a request's keys ends at once, but a grid of
         mostly such blocks still costs time.)"""
         R = len(entries)
-        off, words, T, _, n_rows, host_entries, _, longest, _ = self._pack(entries, bucket, bucket)
+        off, words, T, _, n_rows, host_entries, _, longest, _ = self._pack(entries, bucket, bucket, feed)
         grain = 1024
         while grain * 8 < self.max_model_len:
             grain *= 2
@@ -472,8 +495,7 @@ class StepRunner:
         logit_rows[n_rows:] = 0
         self.rt.copy_h2d_async(self.meta_dev.ptr, self.meta_host.ptr, words * 4)
         self.rt.record(self.meta_copied)
-        if tokens_from is not None:
-            self.rt.copy_d2d(self.meta_dev.ptr + off["tokens"] * 4, tokens_from, R * 4)
+        self._feed(off, tokens_from, R, feed is None)
         picks = self._pick_buffers(bucket) if pick else None
         if self.graph_logits is None and picks is None:
             self.graph_logits = self.rt.empty((self.max_seqs, self.vocab), F32)
@@ -575,7 +597,7 @@ class StepRunner:
         self.steplists[shape] = handle
 
     def step(self, entries: Sequence[StepEntry], download: bool = True, tokens_from: Optional[int] = None,
-             pick: bool = False):
+             pick: bool = False, feed: Optional[Sequence[int]] = None):
         """Run one step.  Returns float32 logits [wanted, vocab] on the host
         (``download=False``: the device tensor, valid until the next step).
         ``pick``: the step wants nothing but the greedy choice of every wanted row; what comes
@@ -585,7 +607,15 @@ class StepRunner:
         ``tokens_from``: a device pointer to int32 token ids, one per entry in the order of the
         entries, for a step in which every entry brings one token: the ids the last step's
         sampling kernel left on the device are fed without a trip to the host (the entries'
-        own token values are then placeholders)."""
+        own token values are then placeholders).  ``feed``: with ``tokens_from``, for any step:
+        per entry the place among those ids that holds the entry's token (the entry then
+        brings one token, a placeholder), or -1 for an entry that brings its tokens itself."""
+        if feed is not None:
+            if tokens_from is None or len(feed) != len(entries):
+                raise ValueError("feed names a place among the ids at tokens_from for every entry, or -1")
+            for e, src in zip(entries, feed):
+                if src >= 0 and len(e.tokens) != 1:
+                    raise ValueError(f"request {e.req!r}: a token fed on the device is one token")
         entries = [e for e in entries if len(e.tokens) > 0]
         if not entries:
             if pick:
@@ -614,22 +644,21 @@ class StepRunner:
             if not m.reserve(e.req, upto):
                 raise OutOfPages(f"request {e.req!r} needs pages for {upto} tokens and the pool "
                                  f"cannot give them: {m.stats()}")
-        if tokens_from is not None and T != R:
-            raise ValueError("tokens_from serves steps in which every request brings one token")
+        if tokens_from is not None and feed is None and T != R:
+            raise ValueError("tokens_from without feed serves steps in which every request brings one token")
         self._clear_untouched(entries)
         self.rt.wait_event(self.meta_copied)     # the last step's copy has left the host buffer
         bucket = self._graph_bucket(entries)
         if bucket:
-            out = self._graph_step(entries, bucket, tokens_from, pick)
+            out = self._graph_step(entries, bucket, tokens_from, pick, feed)
         else:
-            off, words, T, R, n_rows, host_entries, max_q, max_ctx, n_multi = self._pack(entries, T, R)
+            off, words, T, R, n_rows, host_entries, max_q, max_ctx, n_multi = self._pack(entries, T, R, feed)
             picks = self._pick_buffers(n_rows) if pick and n_rows else None
             if picks is None:
                 self._ensure_logits(n_rows)
             self.rt.copy_h2d_async(self.meta_dev.ptr, self.meta_host.ptr, words * 4)
             self.rt.record(self.meta_copied)
-            if tokens_from is not None:
-                self.rt.copy_d2d(self.meta_dev.ptr + off["tokens"] * 4, tokens_from, R * 4)
+            self._feed(off, tokens_from, R, feed is None)
             ctx = self._context(off, T, R, host_entries, max_q, max_ctx, n_multi)
             self.arena.reset()
             if picks is not None:

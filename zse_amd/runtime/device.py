@@ -152,6 +152,7 @@ KERNEL_SIGNATURES = {
     "zk_convert": [_VP, _I, _VP, _I, _SZ, _VP],
     "zk_fill_normal": [_VP, _I, _SZ, _U64, _U64, _F, _F, _VP],
     "zk_zero": [_VP, _SZ, _VP],
+    "zk_feed_tokens": [_VP, _VP, _VP, _VP, _I, _VP],
     "zk_zero_pages": [_VP, _VP, _I, C.POINTER(C.c_int), _I, _VP],
     "zk_gemm_plain": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "zk_attention_plain": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _F,

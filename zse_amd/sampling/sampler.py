@@ -139,43 +139,38 @@ class DeviceSampler:
     """Runs the argmax and inverse-CDF kernels on logits that are still on the device."""
 
     def __init__(self, rt, kernels, max_rows: int):
-        from ..runtime.device import F32, F64, I32
+        from ..runtime.device import F32, F64, I32, Tensor
         self.rt = rt
         self.k = kernels
         self.max_rows = max_rows
         self.ids = rt.empty((max_rows,), I32)
         self.ids2 = rt.empty((max_rows,), I32)
-        self.temp = rt.empty((max_rows,), F32)
-        self.u = rt.empty((max_rows,), F64)
+        # the rows' uniform numbers, shares, temperatures and top-k: one block on the device (24
+        # bytes a row, four arrays of max_rows), so that one copy brings them all
+        self.row_params = rt.empty((max_rows * 6,), F32)
+        base = self.row_params.ptr
+        self.u = Tensor(base, (max_rows,), F64, self.row_params)
+        self.top_p = Tensor(base + max_rows * 8, (max_rows,), F64, self.row_params)
+        self.temp = Tensor(base + max_rows * 16, (max_rows,), F32, self.row_params)
+        self.top_k = Tensor(base + max_rows * 20, (max_rows,), I32, self.row_params)
         self.scratch = rt.empty(((kernels.zk_sample_scratch_bytes(max_rows) + 3) // 4,), F32)
         self.cut_scratch = None                             # histograms and candidates of the cut-offs, on first use
-        self.top_k = rt.empty((max_rows,), I32)
-        self.top_p = rt.empty((max_rows,), F64)
         self._pen = None                                    # (rows, tokens, scales) on the device, grown on demand
-        # the rows' temperatures, uniform numbers and cut-offs on their way to the device: page-locked,
-        # so their copies queue behind the step's kernels instead of waiting for them (``sample``
-        # reads its ids before it returns, so the next call finds the buffer free)
-        self._stage = rt.pinned(max_rows * 24)
-        self._stage_u = self._stage.array(0, max_rows, np.float64)
-        self._stage_p = self._stage.array(max_rows * 8, max_rows, np.float64)
-        self._stage_t = self._stage.array(max_rows * 16, max_rows, np.float32)
-        self._stage_k = self._stage.array(max_rows * 20, max_rows, np.int32)
+        # the same block in page-locked memory, so that its copy queues behind the step's kernels
+        # instead of waiting for them (``sample`` reads its ids before it returns, so the next
+        # call finds the buffer free; steps that do not wait take theirs from a ring)
+        self._stage = self._new_stage()
+        self._ring_stages = None
+        self._ring_stage_at = 0
 
-    # ---- a run of steps without waiting for the host in between
-    RING = 16       # results that may be on their way to the host at a time
+    def _new_stage(self):
+        n = self.max_rows
+        buf = self.rt.pinned(n * 24)
+        return {"buf": buf, "u": buf.array(0, n, np.float64), "p": buf.array(n * 8, n, np.float64),
+                "t": buf.array(n * 16, n, np.float32), "k": buf.array(n * 20, n, np.int32), "event": self.rt.event()}
 
-    @property
-    def run_is_greedy(self) -> bool:
-        """Whether the run that ``prepare_run`` prepared takes the largest logit of every row."""
-        return bool(getattr(self, "_run_greedy", False))
-
-    def can_defer(self, rows: Sequence[dict]) -> bool:
-        """True when ``sample_deferred`` serves these rows: no penalties, and all greedy or all
-        drawn."""
-        if not rows or len(rows) > self.max_rows or not all(r["params"].stateless for r in rows):
-            return False
-        kinds = {bool(r["params"].greedy) for r in rows}
-        return len(kinds) == 1
+    # ---- steps that do not wait for the host
+    RING = 16       # results, and rows' parameters, that may be on their way at a time
 
     # Which kernels a batch needs.  The kernels themselves decide row by row (a top_k of the
     # vocabulary's size or more is no top-k); the host only has to launch the one that serves a
@@ -188,29 +183,58 @@ class DeviceSampler:
     def _is_plain(p: SamplingParams, vocab: Optional[int]) -> bool:
         return p.top_p >= 1.0 and (p.top_k == 0 or vocab is None or p.top_k >= vocab)
 
-    def prepare_run(self, rows: Sequence[dict], us: Sequence[Sequence[float]], vocab: Optional[int] = None):
-        """For a run of steps over the same rows: temperatures once, and the uniform numbers
-        of every step of the run (``us[step][row]``), so that no step of the run copies
-        anything from the host."""
-        from ..runtime.device import F64
+    def can_defer(self, rows: Sequence[dict]) -> bool:
+        """True when ``stage`` and ``sample_staged`` serve these rows: nothing but the logits and
+        a uniform number is needed (no penalty, which looks at the tokens so far)."""
+        return len(rows) <= self.max_rows and all(r["params"].stateless for r in rows)
+
+    def stage(self, rows: Sequence[dict], vocab: Optional[int] = None) -> dict:
+        """Sends the rows' parameters on their way to the device, before the step that makes the
+        logits is even enqueued, so that they are there when it ends.  What comes back goes to
+        ``sample_staged`` with the logits.  A batch that takes the largest logit of every row
+        sends nothing: its step may pick the ids itself (``StepRunner.step(pick=True)``) and hand
+        them to ``ids_deferred``."""
         n = len(rows)
-        self._run_greedy = bool(rows[0]["params"].greedy)
-        if self._run_greedy:
-            return
-        self.rt.copy_h2d(self.temp.ptr, np.array([r["params"].temperature for r in rows], dtype=np.float32))
-        self._run_cut = any(self._has_cut(r["params"], None) for r in rows)
-        self._run_plain = any(self._is_plain(r["params"], vocab) for r in rows)
-        if self._run_cut:
-            self.rt.copy_h2d(self.top_k.ptr, np.array([r["params"].top_k for r in rows], dtype=np.int32))
-            self.rt.copy_h2d(self.top_p.ptr, np.array([r["params"].top_p for r in rows], dtype=np.float64))
-        flat = np.ascontiguousarray(np.asarray(us, dtype=np.float64).reshape(len(us), n))
-        if getattr(self, "_run_u", None) is None or self._run_u.shape[0] < flat.size:
-            self._run_u = self.rt.empty((max(flat.size, self.max_rows * 8),), F64)
-        self.rt.copy_h2d(self._run_u.ptr, flat)
+        greedy = [bool(r["params"].greedy) for r in rows]
+        plan = {"n": n, "all_greedy": all(greedy), "any_greedy": any(greedy), "cut": False, "plain": False}
+        if plan["all_greedy"]:
+            return plan
+        if self._ring_stages is None:
+            self._ring_stages = [self._new_stage() for _ in range(self.RING)]
+        st = self._ring_stages[self._ring_stage_at % self.RING]
+        self._ring_stage_at += 1
+        self.rt.wait_event(st["event"])             # its last copy has left the buffer
+        for i, (r, g) in enumerate(zip(rows, greedy)):
+            p = r["params"]
+            st["t"][i] = 0.0 if g else p.temperature        # a row that is not drawn: the kernels leave it alone
+            st["u"][i] = r["u"]
+            st["k"][i] = p.top_k
+            st["p"][i] = p.top_p
+        plan["cut"] = any(not g and self._has_cut(r["params"], vocab) for r, g in zip(rows, greedy))
+        plan["plain"] = any(not g and self._is_plain(r["params"], vocab) for r, g in zip(rows, greedy))
+        self.rt.copy_h2d_async(self.row_params.ptr, st["buf"].ptr, self.max_rows * 24)
+        self.rt.record(st["event"])
+        return plan
+
+    def sample_staged(self, logits, plan: dict) -> "PendingIds":
+        """Enqueues the sampling of a step whose rows ``stage`` has sent.  The ids stay on the
+        device (``.device_ptr``, valid until the next call) and travel to the host behind the
+        kernels; ``.result()`` waits for them."""
+        n, V = logits.shape
+        if n != plan["n"]:
+            raise ValueError(f"{n} rows of logits for {plan['n']} staged rows")
+        rt, k = self.rt, self.k
+        if plan["all_greedy"]:
+            k.zk_argmax(logits.ptr, self.ids.ptr, n, V, self.scratch.ptr, rt.stream)
+            return self._send(self.ids, n)
+        if plan["any_greedy"]:
+            k.zk_argmax(logits.ptr, self.ids2.ptr, n, V, self.scratch.ptr, rt.stream)
+        self._draw(logits, n, V, self.u.ptr, plan["cut"], plan["plain"])
+        return self._send(self.ids2, n)
 
     def ids_deferred(self, ids) -> "PendingIds":
         """Ids that a step picked itself (``StepRunner.step(pick=True)``, device int32 [n]) on
-        their way to the host: as ``sample_deferred`` of a greedy run, without its kernels."""
+        their way to the host: as ``sample_staged`` of a greedy batch, without its kernels."""
         return self._send(ids, ids.shape[0])
 
     def _send(self, dev, n: int) -> "PendingIds":
@@ -223,20 +247,6 @@ class DeviceSampler:
         rt.copy_d2h_async(host.ptr, dev.ptr, n * 4)
         rt.record(ev)
         return PendingIds(rt, dev.ptr, host, ev, n)
-
-    def sample_deferred(self, logits, step_in_run: int) -> "PendingIds":
-        """Enqueue the sampling of one step of a prepared run.  The ids stay on the device
-        (``.device_ptr``, valid until the next call) and travel to the host behind the
-        kernels; ``.result()`` waits for them."""
-        n, V = logits.shape
-        rt, k = self.rt, self.k
-        if self._run_greedy:
-            k.zk_argmax(logits.ptr, self.ids.ptr, n, V, self.scratch.ptr, rt.stream)
-            dev = self.ids
-        else:
-            self._draw(logits, n, V, self._run_u.ptr + step_in_run * n * 8, self._run_cut, self._run_plain)
-            dev = self.ids2
-        return self._send(dev, n)
 
     def sample(self, logits, rows: Sequence[dict]) -> List[int]:
         """``logits``: device float32 [n, vocab]; ``rows``: per row a dict with
@@ -256,19 +266,15 @@ class DeviceSampler:
         if any(greedy):
             k.zk_argmax(logits.ptr, self.ids.ptr, n, V, self.scratch.ptr, rt.stream)
         if not all(greedy):
-            st = self._stage.ptr
-            self._stage_t[:n] = [1.0 if g else r["params"].temperature for r, g in zip(rows, greedy)]
-            self._stage_u[:n] = [r["u"] for r in rows]
-            rt.copy_h2d_async(self.temp.ptr, st + self.max_rows * 16, n * 4)
-            rt.copy_h2d_async(self.u.ptr, st, n * 8)
+            st = self._stage
+            for i, (r, gr) in enumerate(zip(rows, greedy)):
+                p = r["params"]
+                # (a greedy row goes with temperature 0: the drawing kernels leave it alone)
+                st["t"][i], st["u"][i] = (0.0 if gr else p.temperature), r["u"]
+                st["k"][i], st["p"][i] = p.top_k, p.top_p
             cut = any(not g and self._has_cut(r["params"], V) for r, g in zip(rows, greedy))
             plain = any(not g and self._is_plain(r["params"], V) for r, g in zip(rows, greedy))
-            if cut:
-                # (a greedy row, whose draw nobody reads, as top-k 1: the cheapest there is)
-                self._stage_k[:n] = [1 if g else r["params"].top_k for r, g in zip(rows, greedy)]
-                self._stage_p[:n] = [1.0 if g else r["params"].top_p for r, g in zip(rows, greedy)]
-                rt.copy_h2d_async(self.top_k.ptr, st + self.max_rows * 20, n * 4)
-                rt.copy_h2d_async(self.top_p.ptr, st + self.max_rows * 8, n * 8)
+            rt.copy_h2d_async(self.row_params.ptr, st["buf"].ptr, self.max_rows * 24)
             self._draw(logits, n, V, self.u.ptr, cut, plain)
         g = rt.download(self.ids.rows(0, n)) if any(greedy) else None
         s = rt.download(self.ids2.rows(0, n)) if not all(greedy) else None
