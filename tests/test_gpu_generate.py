@@ -90,6 +90,7 @@ def test_runs_of_steps_without_the_host_give_the_same_tokens(tiny_folders, tempe
         out = [(list(r.output_tokens), r.finish_reason) for r in reqs]
         st = eng.stats()
         assert st.generated_tokens == sum(len(o) for o, _ in out)
+        assert len(st.ttft_ms) == len(reqs) and all(t >= 0 for t in st.ttft_ms + st.tpot_ms)      # every request reported once
         assert all(pool.free_pages == pool.num_pages for pool in eng.runner.manager.pools)
         eng.close()
         return out, st

@@ -93,6 +93,7 @@ class Engine:
         # the last of them left its ids at _last_ids, the row of request r at _last_rows[r]
         self._pending = deque()
         self._last_ids, self._last_rows = None, {}
+        self._ending: Dict[object, Request] = {}     # reached their length in a step whose ids are on their way
 
     def _pages_per_group(self, num_blocks: Optional[int], block_size: int, max_seqs: int, max_len: int,
                          step_tokens: int) -> List[int]:
@@ -247,8 +248,8 @@ class Engine:
         """One step, nothing awaited.  A request's token that the step before has drawn and the
         host has not seen yet is fed to the step on the device; its place in the request's
         output holds a placeholder until the ids arrive (``_resolve``), and the scheduler plans
-        with the numbers of tokens, which it knows.  Returns the requests that reached their
-        length."""
+        with the numbers of tokens, which it knows.  A request that reaches its length here has
+        ended for the scheduler; ``_resolve`` reports it when its last token has been read."""
         sch, runner, sampler = self.scheduler, self.runner, self.sampler
         entries, feed = [], []
         for s in plan.items:
@@ -277,24 +278,37 @@ class Engine:
         else:
             self._last_rows = {}
         self._stats.steps += 1
-        return sch.on_step_done(plan, {r.request_id: None for r, _ in places})
+        for r in sch.on_step_done(plan, {r.request_id: None for r, _ in places}):
+            self._ending[r.request_id] = r           # reached its length: reported when its last token is read
+        return []
 
     def _resolve(self, keep: int) -> List[Request]:
         """Reads the ids of the enqueued steps, oldest first, until at most ``keep`` steps are
         still on their way: puts them where the placeholders are and ends what a stop token
         ends (the request's output is cut back to it; what was computed for it since is thrown
-        away).  Returns the requests that ended so."""
+        away).  Returns the requests whose end is now known in full: by a stop token, or by
+        their length with the last token read.  A request's times are those at which the host
+        had its tokens, not those at which their steps were enqueued."""
         done = []
         while len(self._pending) > keep:
             ids, places = self._pending.popleft()
-            for (r, at), tok in zip(places, ids.result()):
+            toks = ids.result()
+            now = time.monotonic()
+            for (r, at), tok in zip(places, toks):
                 if at >= len(r.output_tokens):          # behind a stop token found in an earlier step
                     continue
                 r.output_tokens[at] = tok
                 self._stats.generated_tokens += 1
+                if at == 0:
+                    r.first_token_time = now
                 if r.params.stop_tokens and tok in r.params.stop_tokens:
-                    if self.scheduler.finish_at(r, at + 1, FinishReason.STOP):
+                    ended_before = self._ending.pop(r.request_id, None) is not None
+                    r.finish_time = None
+                    if self.scheduler.finish_at(r, at + 1, FinishReason.STOP) or ended_before:
                         done.append(r)
+                elif at == len(r.output_tokens) - 1 and self._ending.pop(r.request_id, None) is not None:
+                    r.finish_time = now
+                    done.append(r)
         if done and self._next_plan is not None:
             self._next_plan.items = [s for s in self._next_plan.items if not s.request.finished]
         self._stats.preemptions = self.scheduler.num_preemptions
