@@ -84,9 +84,9 @@ class Engine:
         self._stats = EngineStats()
         self._next_id = 0
         self.quiet = quiet
-        # Steps of single tokens in a row that are enqueued before the host looks at the ids
-        # they produced (1: look after every step).  The ids are fed from step to step on the
-        # device; a stop token found afterwards cuts the request's output back to it.
+        # How many steps may be enqueued before the host looks at the ids of the first of them
+        # (1: it looks after every step).  The ids are fed from step to step on the device; a
+        # stop token found afterwards cuts the request's output back to it.
         self.decode_run = max(1, min(int(decode_run), DeviceSampler.RING))     # results on their way at a time
         self._next_plan: Optional[StepPlan] = None
         # steps whose ids are still on their way: (the ids, [(request, its place in the output)]);
