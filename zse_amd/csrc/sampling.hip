@@ -221,7 +221,9 @@ __global__ __launch_bounds__(256) void sample_pick_kernel(
 //   way 2, whatever is left (more equal logits at the cut-off than the block sorts, both
 //     cut-offs with many candidates, a k-th largest logit 32 below the maximum): the block
 //     narrows a range of keys (the logits' bits, made to sort like the numbers) by eight bits
-//     a pass over the whole row, four passes for top-k and four for top-p, then draws over the row;
+//     a pass over the whole row, four passes for top-k and four for top-p (fewer from the
+//     bucket's own keys on, where the walk found the bucket of a single cut-off), then draws
+//     over the row;
 // A row without cut-offs (way 0) is left alone: zk_sample draws it.
 // (the two zeros are one key: they are equal logits, and which of the equal ones are kept goes
 // by their indices)

@@ -297,7 +297,8 @@ class DeviceSampler:
 
     def cut_ways(self, n: int) -> List[int]:
         """Which way each of the last ``n`` rows drawn with cut-offs went (0: it had none, 1: the
-        candidates, 2: the search over the whole row); for tests and measurements."""
+        candidates down to the cut-off, sorted by one block, 3: the cut-off's bucket sorted and the
+        draw over the whole row, 2: the search over the whole row); for tests and measurements."""
         k = self.k
         words = self.rt.download(self.cut_scratch).view(np.int32)
         at = k.zk_sample_cut_mode_offset() // 4
